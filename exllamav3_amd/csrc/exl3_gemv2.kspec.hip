@@ -54,7 +54,7 @@ __device__ __forceinline__ void static_for(F&& f)
 #define G2_IS_ACT(M) ((M) == G2_MODE_ACT || (M) == G2_MODE_WACT)
 // The modes are separate instantiations because the hot loop needs 62 of the 64 VGPRs that allow two 16-wave workgroups per CU: code
 // of a cold path that is merely present makes the allocator spill (scratch also slows every launch by ~1 us, measured).
-// register budget (waves per SIMD) of an instantiation: chosen so that NO variant spills (tests/test_no_scratch.py)
+// register budget (waves per SIMD) of an instantiation: chosen so that NO variant spills
 constexpr int g2_waves_per_eu(int K, int CB, int NG, int MODE)
 {
     if (MODE == G2_MODE_ACT) return 2;
