@@ -231,3 +231,78 @@ def _declare(l):
     sig("exl3_set_gemm3_cpw", i32)
     sig("exl3_set_attn_wide_waves", i32)
     sig("exl3_set_gemv_defer_wg_per_cu", i32)
+
+
+# ---- the sequence-mixer library (include/exl3_mix.h, csrc/mix_*.hip) -------------------------------------------------------------
+MIX_LIB_PATH = os.path.join(_HERE, "libexl3_mix.so")
+MIX_HEADER_PATH = os.path.join(os.path.dirname(_HERE), "include", "exl3_mix.h")
+MIX_ABI_VERSION = 1
+_mix = None
+
+
+def mix_declared_symbols() -> list[str]:
+    with open(MIX_HEADER_PATH) as f:
+        src = f.read()
+    src = re.sub(r"/\*.*?\*/", "", src, flags=re.S)
+    out = []
+    for n in re.findall(r"\b(exl3_mix_[a-z0-9_]+)\s*\(", src):
+        if n not in out:
+            out.append(n)
+    return out
+
+
+def ensure_mix_built() -> str:
+    """Compile libexl3_mix.so if it is missing or older than its sources (a fresh checkout has no built files; the units of this library
+    take seconds).  Several processes may arrive here at once: the link is written beside the target and renamed over it."""
+    import importlib.util
+    spec = importlib.util.spec_from_file_location("_exl3_build_entry", os.path.join(os.path.dirname(_HERE), "__graft_entry__.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    return mod.build_mix()
+
+
+def mixlib() -> ctypes.CDLL:
+    global _mix
+    if _mix is None:
+        if not os.path.exists(MIX_LIB_PATH):
+            ensure_mix_built()
+        import torch  # noqa: F401      (its HIP runtime first: see lib())
+        _mix = ctypes.CDLL(MIX_LIB_PATH, mode=ctypes.RTLD_GLOBAL)
+        _mix.exl3_mix_last_error.restype = ctypes.c_char_p
+        if _mix.exl3_mix_abi_version() != MIX_ABI_VERSION:
+            raise RuntimeError("exllamav3_amd: libexl3_mix.so is of another ABI version: rebuild with `python __graft_entry__.py`")
+        _declare_mix(_mix)
+    return _mix
+
+
+def check_mix_symbols() -> list[str]:
+    l = mixlib()
+    missing = [s for s in mix_declared_symbols() if not hasattr(l, s)]
+    if missing:
+        raise RuntimeError(f"libexl3_mix.so does not export: {missing}")
+    return mix_declared_symbols()
+
+
+def mix_check(rc: int) -> int:
+    if rc < 0:
+        raise Exl3Error(mixlib().exl3_mix_last_error().decode("utf-8", "replace"))
+    return rc
+
+
+def _declare_mix(l):
+    def sig(name, *argtypes):
+        fn = getattr(l, name)
+        fn.argtypes = list(argtypes)
+        fn.restype = ctypes.c_int
+    sig("exl3_mix_embed", vp, vp, vp, vp, f32, vp, f32, i32, i32, i32, i32, vp)
+    sig("exl3_mix_rms_norm_rows", vp, vp, vp, vp, f32, i32, i32, i32, vp)
+    sig("exl3_mix_gated_residual", vp, vp, i64, vp, i64, vp, vp, f32, i32, i32, i32, vp)
+    sig("exl3_mix_polynorm", vp, vp, i64, vp, f32, i32, i32, i32, vp)
+    sig("exl3_mix_attn_store", vp, vp, vp, vp, i64, vp, i64, vp, vp, vp, vp, f32, i32, i32, i32, i32, i32, i32, vp)
+    sig("exl3_mix_attn_prefill", vp, vp, i64, vp, i64, vp, vp, i64, vp, vp, vp, vp, i32, i32, i32, i32, i32, f32, i32, i32, vp)
+    sig("exl3_mix_attn_decode", vp, vp, i64, vp, vp, vp, i64, vp, vp, vp, i32, i32, i32, i32, i32, f32, i32, i32, vp)
+    sig("exl3_mix_gla_scan", vp, vp, vp, i64, vp, i64, vp, i64, vp, i64, vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, f32, f32, i32, vp)
+    sig("exl3_mix_gla_out", vp, vp, vp, vp, i64, f32, i32, i32, i32, i32, vp)
+    sig("exl3_mix_topk_softmax", vp, vp, vp, i32, i32, i32, vp)
+    sig("exl3_mix_moe_gate_up", vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, vp)
+    sig("exl3_mix_moe_down", vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, vp)

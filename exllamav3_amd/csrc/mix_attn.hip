@@ -1,0 +1,183 @@
+// Sliding-window attention with a learned sink and a head-wise output gate: cache store (value norm, ring buffers) and the exact
+// float32 form of prefill and decode -- one wave per (row, query head), keys of the window across the lanes, an online softmax that
+// starts from the sink.  The matrix-core prefill kernel for bfloat16 lives in mix_attn_mfma.hip; this file is the float32 path and
+// the decode path of both element types.
+#include "mix_common.cuh"
+
+template <typename T>
+__global__ __launch_bounds__(64) void attn_store_kernel(T* __restrict__ v_norm, T* __restrict__ ring_k, T* __restrict__ ring_v, const T* __restrict__ k, int64_t k_ld,
+                                                        const T* __restrict__ v, int64_t v_ld, const int32_t* __restrict__ tok_seq,
+                                                        const int32_t* __restrict__ tok_pos, const int32_t* __restrict__ slots,
+                                                        const int32_t* __restrict__ len_after, float eps, int kv_heads, int dim, int vdim, int window)
+{
+    const int n = blockIdx.x, g = blockIdx.y, lane = threadIdx.x;
+    const T* vr = v + (int64_t) n * v_ld + (int64_t) g * vdim;
+    float ss = 0.f;
+    for (int i = lane; i < vdim; i += 64) { float x = to_f(vr[i]); ss += x * x; }
+    ss = wave_sum(ss);
+    const float inv = 1.0f / sqrtf(ss / (float) vdim + eps);
+    const int b = tok_seq[n], pos = tok_pos[n];
+    const bool keep = pos >= len_after[b] - window;
+    const int64_t slot_row = ((int64_t) slots[b] * window + (pos % window)) * kv_heads + g;
+    T* vn = v_norm + ((int64_t) n * kv_heads + g) * vdim;
+    T* rv = ring_v + slot_row * vdim;
+    for (int i = lane; i < vdim; i += 64)
+    {
+        T o = from_f<T>(to_f(vr[i]) * inv);
+        vn[i] = o;
+        if (keep) rv[i] = o;
+    }
+    if (keep)
+    {
+        const T* kr = k + (int64_t) n * k_ld + (int64_t) g * dim;
+        T* rk = ring_k + slot_row * dim;
+        for (int i = lane; i < dim; i += 64) rk[i] = kr[i];
+    }
+}
+
+// One wave per (row, head).  Keys kb + j * k_step, values vb + j * v_step, j < count.  MAXV = ceil(vdim / 64) accumulators per lane.
+template <typename T, int MAXV>
+__device__ __forceinline__ void attn_row(T* __restrict__ out, const T* __restrict__ q, const T* __restrict__ kb, int64_t k_step, const T* __restrict__ vb,
+                                         int64_t v_step, int count, int dim, int vdim, float scale, bool has_sink, float sink, float gate,
+                                         float* qs, float* ps)
+{
+    const int lane = threadIdx.x;
+    for (int i = lane; i < dim; i += 64) qs[i] = to_f(q[i]);
+    __syncthreads();
+    float m = has_sink ? sink : -INFINITY, l = has_sink ? 1.0f : 0.0f;
+    float acc[MAXV];
+    #pragma unroll
+    for (int i = 0; i < MAXV; ++i) acc[i] = 0.f;
+    for (int j0 = 0; j0 < count; j0 += 64)
+    {
+        const int j = j0 + lane;
+        float s = -INFINITY;
+        if (j < count)
+        {
+            const T* kr = kb + (int64_t) j * k_step;
+            float d = 0.f;
+            for (int c = 0; c < dim; ++c) d += qs[c] * to_f(kr[c]);
+            s = d * scale;
+        }
+        const float m_new = fmaxf(m, wave_max(s));          // finite: j0 < count, so lane 0 of the chunk holds a score
+        const float p = (j < count) ? expf(s - m_new) : 0.f;
+        const float corr = expf(m - m_new);                 // m = -inf (no sink, first chunk): 0
+        l = l * corr + wave_sum(p);
+        m = m_new;
+        __syncthreads();
+        ps[lane] = p;
+        __syncthreads();
+        const int cnt = min(64, count - j0);
+        #pragma unroll
+        for (int i = 0; i < MAXV; ++i)
+        {
+            const int c = lane + 64 * i;
+            float a = acc[i] * corr;
+            if (c < vdim)
+                for (int jj = 0; jj < cnt; ++jj) a += ps[jj] * to_f(vb[(int64_t) (j0 + jj) * v_step + c]);
+            acc[i] = a;
+        }
+    }
+    const float f = (l > 0.f ? 1.0f / l : 0.f) * gate;
+    #pragma unroll
+    for (int i = 0; i < MAXV; ++i)
+    {
+        const int c = lane + 64 * i;
+        if (c < vdim) out[c] = from_f<T>(acc[i] * f);
+    }
+}
+
+template <typename T, int MAXV>
+__global__ __launch_bounds__(64) void attn_prefill_kernel(T* __restrict__ out, const T* __restrict__ q, int64_t q_ld, const T* __restrict__ k, int64_t k_ld,
+                                                          const T* __restrict__ v_norm, const T* __restrict__ gate, int64_t gate_ld, const float* __restrict__ sink,
+                                                          const int32_t* __restrict__ cu, const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ tok_pos,
+                                                          int heads, int kv_heads, int dim, int vdim, float scale, int window)
+{
+    extern __shared__ float smem[];
+    float* qs = smem; float* ps = smem + dim;
+    const int n = blockIdx.x, h = blockIdx.y;
+    const int g = h / (heads / kv_heads);
+    const int b = tok_seq[n], first = cu[b];
+    const int i = n - first;                                  // the row's place in its sequence == its position (the sequence starts in this step)
+    const int lo = max(0, i - window + 1);
+    const float gt = gate ? sigmoid_f(to_f(gate[(int64_t) n * gate_ld + h])) : 1.0f;
+    attn_row<T, MAXV>(out + ((int64_t) n * heads + h) * vdim, q + (int64_t) n * q_ld + (int64_t) h * dim,
+                      k + (int64_t) (first + lo) * k_ld + (int64_t) g * dim, k_ld,
+                      v_norm + ((int64_t) (first + lo) * kv_heads + g) * vdim, (int64_t) kv_heads * vdim,
+                      i - lo + 1, dim, vdim, scale, sink != nullptr, sink ? sink[h] : 0.f, gt, qs, ps);
+}
+
+template <typename T, int MAXV>
+__global__ __launch_bounds__(64) void attn_decode_kernel(T* __restrict__ out, const T* __restrict__ q, int64_t q_ld, const T* __restrict__ ring_k,
+                                                         const T* __restrict__ ring_v, const T* __restrict__ gate, int64_t gate_ld, const float* __restrict__ sink,
+                                                         const int32_t* __restrict__ slots, const int32_t* __restrict__ len_after,
+                                                         int heads, int kv_heads, int dim, int vdim, float scale, int window)
+{
+    extern __shared__ float smem[];
+    float* qs = smem; float* ps = smem + dim;
+    const int n = blockIdx.x, h = blockIdx.y;
+    const int g = h / (heads / kv_heads);
+    const int count = min(len_after[n], window);
+    const int64_t base = (int64_t) slots[n] * window * kv_heads + g;
+    const float gt = gate ? sigmoid_f(to_f(gate[(int64_t) n * gate_ld + h])) : 1.0f;
+    attn_row<T, MAXV>(out + ((int64_t) n * heads + h) * vdim, q + (int64_t) n * q_ld + (int64_t) h * dim,
+                      ring_k + base * dim, (int64_t) kv_heads * dim, ring_v + base * vdim, (int64_t) kv_heads * vdim,
+                      count, dim, vdim, scale, sink != nullptr, sink ? sink[h] : 0.f, gt, qs, ps);
+}
+
+extern "C" int exl3_mix_attn_store(void* v_norm, void* ring_k, void* ring_v, const void* k, int64_t k_ld, const void* v, int64_t v_ld,
+                                   const int32_t* tok_seq, const int32_t* tok_pos, const int32_t* slots, const int32_t* len_after,
+                                   float eps, int n, int kv_heads, int dim, int vdim, int window, int dtype, void* stream)
+{
+    MIX_CHECK(v_norm && ring_k && ring_v && k && v && tok_seq && tok_pos && slots && len_after, "mix_attn_store: null pointer");
+    MIX_CHECK(n >= 0 && kv_heads > 0 && dim > 0 && vdim > 0 && window > 0 && k_ld >= (int64_t) kv_heads * dim && v_ld >= (int64_t) kv_heads * vdim,
+              "mix_attn_store: bad sizes");
+    if (n == 0) return EXL3_MIX_OK;
+    MIX_DISPATCH_T(dtype, hipLaunchKernelGGL(attn_store_kernel<T>, dim3(n, kv_heads), dim3(64), 0, (hipStream_t) stream, (T*) v_norm, (T*) ring_k, (T*) ring_v,
+                                             (const T*) k, k_ld, (const T*) v, v_ld, tok_seq, tok_pos, slots, len_after, eps, kv_heads, dim, vdim, window));
+    return mix_check_launch("mix_attn_store");
+}
+
+#define ATTN_LAUNCH(KERNEL, ...) \
+    do { \
+        const size_t sm = (size_t) (dim + 64) * sizeof(float); \
+        const int mv = (vdim + 63) / 64; \
+        MIX_DISPATCH_T(dtype, \
+            if (mv == 1)      hipLaunchKernelGGL((KERNEL<T, 1>), dim3(n, heads), dim3(64), sm, (hipStream_t) stream, __VA_ARGS__); \
+            else if (mv == 2) hipLaunchKernelGGL((KERNEL<T, 2>), dim3(n, heads), dim3(64), sm, (hipStream_t) stream, __VA_ARGS__); \
+            else if (mv <= 4) hipLaunchKernelGGL((KERNEL<T, 4>), dim3(n, heads), dim3(64), sm, (hipStream_t) stream, __VA_ARGS__); \
+            else              hipLaunchKernelGGL((KERNEL<T, 8>), dim3(n, heads), dim3(64), sm, (hipStream_t) stream, __VA_ARGS__)); \
+    } while (0)
+
+static int attn_check(const char* what, int n, int heads, int kv_heads, int dim, int vdim, int window)
+{
+    MIX_CHECK(n >= 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0, "%s: heads %d must be a multiple of kv_heads %d", what, heads, kv_heads);
+    MIX_CHECK(dim > 0 && dim <= 4096 && vdim > 0 && vdim <= 512 && window > 0, "%s: dim %d / vdim %d / window %d out of range", what, dim, vdim, window);
+    return EXL3_MIX_OK;
+}
+
+extern "C" int exl3_mix_attn_prefill(void* out, const void* q, int64_t q_ld, const void* k, int64_t k_ld, const void* v_norm,
+                                     const void* gate, int64_t gate_ld, const float* sink, const int32_t* cu, const int32_t* tok_seq, const int32_t* tok_pos,
+                                     int n, int heads, int kv_heads, int dim, int vdim, float scale, int window, int dtype, void* stream)
+{
+    MIX_CHECK(out && q && k && v_norm && cu && tok_seq && tok_pos, "mix_attn_prefill: null pointer");
+    if (int rc = attn_check("mix_attn_prefill", n, heads, kv_heads, dim, vdim, window)) return rc;
+    MIX_CHECK(q_ld >= (int64_t) heads * dim && k_ld >= (int64_t) kv_heads * dim && (!gate || gate_ld >= heads), "mix_attn_prefill: bad row strides");
+    if (n == 0) return EXL3_MIX_OK;
+    ATTN_LAUNCH(attn_prefill_kernel, (T*) out, (const T*) q, q_ld, (const T*) k, k_ld, (const T*) v_norm, (const T*) gate, gate_ld, sink, cu, tok_seq, tok_pos,
+                heads, kv_heads, dim, vdim, scale, window);
+    return mix_check_launch("mix_attn_prefill");
+}
+
+extern "C" int exl3_mix_attn_decode(void* out, const void* q, int64_t q_ld, const void* ring_k, const void* ring_v,
+                                    const void* gate, int64_t gate_ld, const float* sink, const int32_t* slots, const int32_t* len_after,
+                                    int n, int heads, int kv_heads, int dim, int vdim, float scale, int window, int dtype, void* stream)
+{
+    MIX_CHECK(out && q && ring_k && ring_v && slots && len_after, "mix_attn_decode: null pointer");
+    if (int rc = attn_check("mix_attn_decode", n, heads, kv_heads, dim, vdim, window)) return rc;
+    MIX_CHECK(q_ld >= (int64_t) heads * dim && (!gate || gate_ld >= heads), "mix_attn_decode: bad row strides");
+    if (n == 0) return EXL3_MIX_OK;
+    ATTN_LAUNCH(attn_decode_kernel, (T*) out, (const T*) q, q_ld, (const T*) ring_k, (const T*) ring_v, (const T*) gate, gate_ld, sink, slots, len_after,
+                heads, kv_heads, dim, vdim, scale, window);
+    return mix_check_launch("mix_attn_decode");
+}

@@ -1,0 +1,66 @@
+// Device helpers of the sequence-mixer library (libexl3_mix.so): element types, conversions, reductions.  gfx950 only (wave64).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdarg.h>
+#include <stdio.h>
+#include "../../include/exl3_mix.h"
+
+struct bf16_t { uint16_t u; };
+
+__device__ __forceinline__ float to_f(bf16_t v) { return __uint_as_float(((uint32_t) v.u) << 16); }
+__device__ __forceinline__ float to_f(float v) { return v; }
+
+template <typename T> __device__ __forceinline__ T from_f(float f);
+template <> __device__ __forceinline__ bf16_t from_f<bf16_t>(float f)
+{
+    uint32_t u = __float_as_uint(f);
+    bf16_t r;
+    if ((u & 0x7fffffffu) > 0x7f800000u) { r.u = 0x7fc0; return r; }
+    u += 0x7fffu + ((u >> 16) & 1u);                 // round to nearest, ties to even
+    r.u = (uint16_t) (u >> 16);
+    return r;
+}
+template <> __device__ __forceinline__ float from_f<float>(float f) { return f; }
+
+__device__ __forceinline__ float wave_sum(float v)
+{
+    #pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+__device__ __forceinline__ float wave_max(float v)
+{
+    #pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+    return v;
+}
+
+// sum over a workgroup of NW waves; every thread gets the result.  `red` holds NW floats; two barriers.
+template <int NW>
+__device__ __forceinline__ float block_sum(float v, float* red)
+{
+    v = wave_sum(v);
+    const int w = threadIdx.x >> 6;
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) red[w] = v;
+    __syncthreads();
+    float s = 0.f;
+    #pragma unroll
+    for (int i = 0; i < NW; ++i) s += red[i];
+    return s;
+}
+
+__device__ __forceinline__ float sigmoid_f(float z) { return 1.0f / (1.0f + expf(-z)); }
+__device__ __forceinline__ float silu_f(float z) { return z / (1.0f + expf(-z)); }
+// log(sigmoid(z)) without cancellation on either side
+__device__ __forceinline__ float log_sigmoid_f(float z) { return fminf(z, 0.f) - log1pf(expf(-fabsf(z))); }
+
+// error reporting shared by the translation units of this library (thread-local message, negative return codes)
+void mix_set_error(const char* fmt, ...);
+int  mix_check_launch(const char* what);
+#define MIX_CHECK(cond, ...) do { if (!(cond)) { mix_set_error(__VA_ARGS__); return EXL3_MIX_ERR_ARG; } } while (0)
+
+// dispatch on the activation element type: 0 = bfloat16, 1 = float32
+#define MIX_DISPATCH_T(dtype, ...) \
+    do { if ((dtype) == EXL3_MIX_BF16) { using T = bf16_t; __VA_ARGS__; } else { using T = float; __VA_ARGS__; } } while (0)

@@ -1,0 +1,176 @@
+"""
+Python surface of the sequence-mixer library libexl3_mix.so (include/exl3_mix.h): one function per kernel, torch tensors in, raw device
+pointers out, on the caller's current HIP stream.  PyTorch is device memory and streams only; there is no eager or CPU fallback -- a
+missing library is compiled on first use (seconds) and anything else raises.
+
+Activations and matrix weights are bfloat16 or float32 (`code(dtype)`); the residual stream, norm weights, sinks, decay biases, recurrent
+states and router logits are float32 in both modes.  2-D arguments named *_view may be column blocks of a wider matrix (unit column
+stride, any row stride).
+"""
+from __future__ import annotations
+import torch
+from . import _lib
+from ._lib import mix_check as _check
+
+BF16, F32 = 0, 1
+
+
+def code(dtype: torch.dtype) -> int:
+    if dtype == torch.bfloat16:
+        return BF16
+    if dtype == torch.float32:
+        return F32
+    raise RuntimeError(f"mix_ops: activations are bfloat16 or float32, not {dtype}")
+
+
+def _p(t):
+    return None if t is None else t.data_ptr()
+
+
+def _stream(t: torch.Tensor):
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _req(cond, msg):
+    if not cond:
+        raise RuntimeError(msg)
+
+
+def _view(t: torch.Tensor, cols: int, name: str) -> int:
+    """Row stride of a 2-D column block."""
+    _req(t.dim() == 2 and t.shape[1] == cols and (t.stride(1) == 1 or cols == 1), f"{name}: expected [rows, {cols}] with unit column stride, got {tuple(t.shape)} / {t.stride()}")
+    return t.stride(0)
+
+
+def _f32c(t: torch.Tensor, name: str):
+    _req(t.dtype == torch.float32 and t.is_contiguous(), f"{name}: contiguous float32 expected")
+
+
+def _i32c(t: torch.Tensor, name: str):
+    _req(t.dtype == torch.int32 and t.is_contiguous(), f"{name}: contiguous int32 expected")
+
+
+def embed(x: torch.Tensor, h: torch.Tensor | None, table: torch.Tensor, tokens: torch.Tensor, scale: float, norm_w: torch.Tensor | None, eps: float):
+    n, width = x.shape
+    _f32c(x, "x"); _i32c(tokens, "tokens")
+    _req(tokens.numel() == n and table.is_contiguous() and table.shape[1] == width, "embed: shapes")
+    if norm_w is not None:
+        _f32c(norm_w, "norm_w"); _req(h is not None and h.is_contiguous() and h.shape == x.shape and h.dtype == table.dtype, "embed: h")
+    _check(_lib.mixlib().exl3_mix_embed(_p(x), _p(h), _p(table), _p(tokens), scale, _p(norm_w), eps, n, width, table.shape[0], code(table.dtype), _stream(x)))
+
+
+def rms_norm_rows(h: torch.Tensor, x: torch.Tensor, rows: torch.Tensor | None, w: torch.Tensor, eps: float):
+    n, width = h.shape
+    _f32c(x, "x"); _f32c(w, "w")
+    _req(h.is_contiguous() and x.shape[1] == width and w.numel() == width, "rms_norm_rows: shapes")
+    if rows is not None:
+        _i32c(rows, "rows"); _req(rows.numel() == n, "rms_norm_rows: rows")
+    else:
+        _req(x.shape[0] == n, "rms_norm_rows: rows of x")
+    _check(_lib.mixlib().exl3_mix_rms_norm_rows(_p(h), _p(x), _p(rows), _p(w), eps, n, width, code(h.dtype), _stream(x)))
+
+
+def gated_residual(x: torch.Tensor, y_view: torch.Tensor, r_view: torch.Tensor, norm_w: torch.Tensor | None, h: torch.Tensor | None, eps: float):
+    n, width = x.shape
+    _f32c(x, "x")
+    _req(y_view.dtype == r_view.dtype and y_view.shape[0] == n and r_view.shape[0] == n, "gated_residual: y / r")
+    if norm_w is not None:
+        _f32c(norm_w, "norm_w"); _req(h is not None and h.is_contiguous() and h.shape == x.shape and h.dtype == y_view.dtype, "gated_residual: h")
+    _check(_lib.mixlib().exl3_mix_gated_residual(_p(x), _p(y_view), _view(y_view, width, "y"), _p(r_view), _view(r_view, width, "r"), _p(norm_w), _p(h), eps, n, width,
+                                                  code(y_view.dtype), _stream(x)))
+
+
+def polynorm(out: torch.Tensor, z_view: torch.Tensor, coef: torch.Tensor, eps: float):
+    n, ff = out.shape
+    _f32c(coef, "coef")
+    _req(out.is_contiguous() and z_view.dtype == out.dtype and z_view.shape[0] == n and coef.numel() == 4, "polynorm: shapes")
+    _check(_lib.mixlib().exl3_mix_polynorm(_p(out), _p(z_view), _view(z_view, ff, "z"), _p(coef), eps, n, ff, code(out.dtype), _stream(out)))
+
+
+def attn_store(v_norm, ring_k, ring_v, k_view, v_view, tok_seq, tok_pos, slots, len_after, eps: float):
+    n, kv_heads, vdim = v_norm.shape
+    n_slots, window, g2, dim = ring_k.shape
+    _req(g2 == kv_heads and ring_v.shape == (n_slots, window, kv_heads, vdim) and ring_k.is_contiguous() and ring_v.is_contiguous() and v_norm.is_contiguous(),
+         "attn_store: cache shapes")
+    _req(ring_k.dtype == k_view.dtype == v_view.dtype == v_norm.dtype == ring_v.dtype, "attn_store: element types")
+    for t, nm in ((tok_seq, "tok_seq"), (tok_pos, "tok_pos"), (slots, "slots"), (len_after, "len_after")):
+        _i32c(t, nm)
+    _req(tok_seq.numel() == n and tok_pos.numel() == n and k_view.shape[0] == n and v_view.shape[0] == n, "attn_store: rows")
+    _check(_lib.mixlib().exl3_mix_attn_store(_p(v_norm), _p(ring_k), _p(ring_v), _p(k_view), _view(k_view, kv_heads * dim, "k"), _p(v_view),
+                                              _view(v_view, kv_heads * vdim, "v"), _p(tok_seq), _p(tok_pos), _p(slots), _p(len_after), eps, n, kv_heads, dim, vdim, window,
+                                              code(v_norm.dtype), _stream(v_norm)))
+
+
+def attn_prefill(out, q_view, k_view, v_norm, gate_view, sink, cu, tok_seq, tok_pos, heads: int, scale: float, window: int):
+    n, kv_heads, vdim = v_norm.shape
+    dim = q_view.shape[1] // heads
+    _req(out.is_contiguous() and out.shape == (n, heads * vdim) and out.dtype == q_view.dtype == k_view.dtype == v_norm.dtype, "attn_prefill: out / types")
+    if sink is not None:
+        _f32c(sink, "sink"); _req(sink.numel() == heads, "attn_prefill: sink")
+    _check(_lib.mixlib().exl3_mix_attn_prefill(_p(out), _p(q_view), _view(q_view, heads * dim, "q"), _p(k_view), _view(k_view, kv_heads * dim, "k"), _p(v_norm),
+                                                _p(gate_view), 0 if gate_view is None else _view(gate_view, heads, "gate"), _p(sink), _p(cu), _p(tok_seq), _p(tok_pos),
+                                                n, heads, kv_heads, dim, vdim, scale, window, code(out.dtype), _stream(out)))
+
+
+def attn_decode(out, q_view, ring_k, ring_v, gate_view, sink, slots, len_after, heads: int, scale: float):
+    n = out.shape[0]
+    n_slots, window, kv_heads, dim = ring_k.shape
+    vdim = ring_v.shape[3]
+    _req(out.is_contiguous() and out.shape == (n, heads * vdim) and out.dtype == q_view.dtype == ring_k.dtype, "attn_decode: out / types")
+    _req(slots.numel() == n and len_after.numel() == n, "attn_decode: one row per sequence")
+    if sink is not None:
+        _f32c(sink, "sink"); _req(sink.numel() == heads, "attn_decode: sink")
+    _check(_lib.mixlib().exl3_mix_attn_decode(_p(out), _p(q_view), _view(q_view, heads * dim, "q"), _p(ring_k), _p(ring_v), _p(gate_view),
+                                               0 if gate_view is None else _view(gate_view, heads, "gate"), _p(sink), _p(slots), _p(len_after),
+                                               n, heads, kv_heads, dim, vdim, scale, window, code(out.dtype), _stream(out)))
+
+
+def gla_scan(o, state, q_view, k_view, v_view, lr_view, a2, a2_bias, cu, slots, pos0, tau: float, q_scale: float, chunked: bool = False):
+    n, heads, vdim = o.shape
+    n_slots, h2, dim, v2 = state.shape
+    rank = a2.shape[1]
+    _f32c(o, "o"); _f32c(state, "state")
+    _req(h2 == heads and v2 == vdim and a2.is_contiguous() and a2.shape[0] == heads * dim and a2.dtype == q_view.dtype, "gla_scan: shapes")
+    if a2_bias is not None:
+        _f32c(a2_bias, "a2_bias")
+    batch = slots.numel()
+    _req(cu.numel() == batch + 1 and pos0.numel() == batch, "gla_scan: batch tensors")
+    fn = _lib.mixlib().exl3_mix_gla_chunked if chunked else _lib.mixlib().exl3_mix_gla_scan
+    _check(fn(_p(o), _p(state), _p(q_view), _view(q_view, heads * dim, "q"), _p(k_view), _view(k_view, heads * dim, "k"), _p(v_view),
+              _view(v_view, heads * vdim, "v"), _p(lr_view), _view(lr_view, rank, "lr"), _p(a2), _p(a2_bias), _p(cu), _p(slots), _p(pos0),
+              batch, heads, dim, vdim, rank, tau, q_scale, code(q_view.dtype), _stream(o)))
+
+
+def gla_out(out, o, w, g_view, eps: float):
+    n, heads, vdim = o.shape
+    _f32c(o, "o"); _f32c(w, "w")
+    _req(out.is_contiguous() and out.shape == (n, heads * vdim) and w.numel() == vdim and g_view.dtype == out.dtype, "gla_out: shapes")
+    _check(_lib.mixlib().exl3_mix_gla_out(_p(out), _p(o), _p(w), _p(g_view), _view(g_view, heads * vdim, "g"), eps, n, heads, vdim, code(out.dtype), _stream(out)))
+
+
+def topk_softmax(idx, wts, logits):
+    n, experts = logits.shape
+    top = idx.shape[1]
+    _f32c(logits, "logits"); _f32c(wts, "wts"); _i32c(idx, "idx")
+    _req(idx.shape == wts.shape == (n, top), "topk_softmax: shapes")
+    _check(_lib.mixlib().exl3_mix_topk_softmax(_p(idx), _p(wts), _p(logits), n, experts, top, _stream(logits)))
+
+
+def moe_gate_up(hid, h, wg, wu, idx):
+    n, width = h.shape
+    experts, ff, w2 = wg.shape
+    top = idx.shape[1]
+    _req(h.is_contiguous() and wg.is_contiguous() and wu.is_contiguous() and wu.shape == wg.shape and w2 == width and hid.is_contiguous()
+         and hid.shape == (n * top, ff) and hid.dtype == h.dtype == wg.dtype, "moe_gate_up: shapes")
+    _i32c(idx, "idx")
+    _check(_lib.mixlib().exl3_mix_moe_gate_up(_p(hid), _p(h), _p(wg), _p(wu), _p(idx), n, top, experts, ff, width, code(h.dtype), _stream(h)))
+
+
+def moe_down(y, hid, wd, idx, wts):
+    n, width = y.shape
+    experts, w2, ff = wd.shape
+    top = idx.shape[1]
+    _req(y.is_contiguous() and hid.is_contiguous() and wd.is_contiguous() and w2 == width and hid.shape == (n * top, ff) and y.dtype == hid.dtype == wd.dtype,
+         "moe_down: shapes")
+    _i32c(idx, "idx"); _f32c(wts, "wts")
+    _check(_lib.mixlib().exl3_mix_moe_down(_p(y), _p(hid), _p(wd), _p(idx), _p(wts), n, top, experts, ff, width, code(y.dtype), _stream(y)))

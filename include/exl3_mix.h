@@ -1,0 +1,103 @@
+/*
+ * exl3_mix.h -- C-ABI of the sequence-mixer library (libexl3_mix.so): the kernels of models whose layers are not the
+ * quantized-linear transformer block of libexl3_hip.so -- sliding-window attention with a learned sink over a ring cache, gated
+ * linear attention with a per-channel decay and a carried state, RMS norms over a 32-bit residual stream, a gated residual,
+ * the PolyNorm activation, a top-k router and unquantized experts.
+ *
+ * Conventions (the same as exl3_hip.h): plain device pointers, sizes and scalars; `stream` is a hipStream_t; calls are
+ * asynchronous; return 0 on success and < 0 on error with the text in exl3_mix_last_error() (thread-local).
+ *
+ *   - `dtype` names the element type of activations and of matrix weights: EXL3_MIX_BF16 or EXL3_MIX_F32.  The residual stream,
+ *     norm weights, biases read by these kernels, sinks, decay biases, recurrent states, scores and softmax weights are float32
+ *     in both modes.
+ *   - A step's tokens are PACKED: N rows, the sequences of a batch one behind the other without padding.  cu[b] .. cu[b+1] are the
+ *     rows of sequence b; tok_seq[n] / tok_pos[n] give a row's sequence and its position in that sequence (counted from 0 over the
+ *     sequence's whole life, not over the step).  slots[b] is the sequence's slot in the state buffers.
+ *   - A row stride `*_ld` counts elements between consecutive rows, so that a kernel reads a column block of a wider matrix product
+ *     in place.
+ */
+#ifndef EXL3_MIX_H
+#define EXL3_MIX_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define EXL3_MIX_OK        0
+#define EXL3_MIX_ERR_ARG  (-1)
+#define EXL3_MIX_ERR_HIP  (-2)
+
+#define EXL3_MIX_BF16 0
+#define EXL3_MIX_F32  1
+
+#define EXL3_MIX_ABI_VERSION 1
+
+const char* exl3_mix_last_error(void);
+int  exl3_mix_abi_version(void);
+
+/* x[n] = table[tokens[n]] * scale (float32 residual);  if norm_w: h[n] = x[n] / sqrt(mean(x[n]^2) + eps) * norm_w. */
+int exl3_mix_embed(float* x, void* h, const void* table, const int32_t* tokens, float scale, const float* norm_w, float eps,
+                   int n, int width, int vocab, int dtype, void* stream);
+
+/* h[i] = rms_norm(x[rows ? rows[i] : i]) * w: RMS norm of selected residual rows (the model's last norm runs on the wanted rows only). */
+int exl3_mix_rms_norm_rows(void* h, const float* x, const int32_t* rows, const float* w, float eps, int n, int width, int dtype, void* stream);
+
+/* Gated residual: x[n] += y[n] * sigmoid(r[n])  (r holds the gate's pre-activation, bias included), then, if norm_w, the next
+ * sublayer's input h[n] = rms_norm(x[n]) * norm_w.  y and r are column blocks of wider matrices (row strides y_ld, r_ld). */
+int exl3_mix_gated_residual(float* x, const void* y, int64_t y_ld, const void* r, int64_t r_ld, const float* norm_w, void* h, float eps,
+                            int n, int width, int dtype, void* stream);
+
+/* PolyNorm: out = a N(z) + b N(z^2) + c N(z^3) + e with N(u) = u / sqrt(mean(u^2) + eps) over a row; coef = {a, b, c, e} (float32, device). */
+int exl3_mix_polynorm(void* out, const void* z, int64_t z_ld, const float* coef, float eps, int n, int ff, int dtype, void* stream);
+
+/* Values of a step enter the attention cache: every key/value head's value is divided by its root mean square (eps inside the
+ * root, no weight) and written to v_norm [n][kv_heads][vdim]; keys and normalised values of the rows that are among the last
+ * `window` positions of their sequence (tok_pos >= len_after[seq] - window) go to the ring buffers
+ * ring_k [slots][window][kv_heads][dim], ring_v [slots][window][kv_heads][vdim] at position tok_pos % window. */
+int exl3_mix_attn_store(void* v_norm, void* ring_k, void* ring_v, const void* k, int64_t k_ld, const void* v, int64_t v_ld,
+                        const int32_t* tok_seq, const int32_t* tok_pos, const int32_t* slots, const int32_t* len_after,
+                        float eps, int n, int kv_heads, int dim, int vdim, int window, int dtype, void* stream);
+
+/* Sliding-window attention with a sink over the step's own keys (sequences that start at position 0 in this step):
+ * row i sees rows j of its sequence with 0 <= i - j < window; weights = exp(s_j - m) / (exp(sink_h - m) + sum_j exp(s_j - m)),
+ * s_j = scale * q.k_j; out[n][h] = sigmoid(gate[n][h]) * sum_j w_j v_j.  sink may be NULL (plain softmax), gate may be NULL.
+ * v_norm as written by exl3_mix_attn_store.  Scores, weights and sums are float32. */
+int exl3_mix_attn_prefill(void* out, const void* q, int64_t q_ld, const void* k, int64_t k_ld, const void* v_norm,
+                          const void* gate, int64_t gate_ld, const float* sink, const int32_t* cu, const int32_t* tok_seq, const int32_t* tok_pos,
+                          int n, int heads, int kv_heads, int dim, int vdim, float scale, int window, int dtype, void* stream);
+
+/* The same for one new row per sequence against the ring buffers (which already hold the row's own key and value):
+ * row b sees the min(len_after[b], window) newest entries of slot slots[b]. */
+int exl3_mix_attn_decode(void* out, const void* q, int64_t q_ld, const void* ring_k, const void* ring_v,
+                         const void* gate, int64_t gate_ld, const float* sink, const int32_t* slots, const int32_t* len_after,
+                         int n, int heads, int kv_heads, int dim, int vdim, float scale, int window, int dtype, void* stream);
+
+/* Gated linear attention, token by token (prefill of any length and decode): per sequence b and head h, with the state S [dim][vdim]
+ * (float32, state [slots][heads][dim][vdim]; taken as zero where pos0[b] == 0, read from slot slots[b] otherwise, written back at the end):
+ *     alpha_t = exp(log_sigmoid(z_t) / tau),  z_t = a2 . lr_t + a2_bias      (lr: the low-rank decay input [n][rank], a2 [heads*dim][rank])
+ *     S <- diag(alpha_t) S + k_t v_t^T,   o_t = S^T (q_t * q_scale)
+ * o [n][heads][vdim] float32. */
+int exl3_mix_gla_scan(float* o, float* state, const void* q, int64_t q_ld, const void* k, int64_t k_ld, const void* v, int64_t v_ld,
+                      const void* lr, int64_t lr_ld, const void* a2, const float* a2_bias, const int32_t* cu, const int32_t* slots, const int32_t* pos0,
+                      int batch, int heads, int dim, int vdim, int rank, float tau, float q_scale, int dtype, void* stream);
+
+/* out[n][h*vdim + v] = o[n][h][v] / sqrt(mean_v(o[n][h]^2) + eps) * w[v] * silu(g[n][h*vdim + v]) */
+int exl3_mix_gla_out(void* out, const float* o, const float* w, const void* g, int64_t g_ld, float eps, int n, int heads, int vdim, int dtype, void* stream);
+
+/* Router: the `top` largest of `experts` logits per row (float32; ties go to the lower index), weights = softmax over the chosen logits. */
+int exl3_mix_topk_softmax(int32_t* idx, float* wts, const float* logits, int n, int experts, int top, void* stream);
+
+/* Experts of a few rows, weights streamed once per (row, choice): hid[n*top + r] = silu(Wg[e] h[n]) * (Wu[e] h[n]) with e = idx[n][r];
+ * Wg, Wu [experts][ff][width]. */
+int exl3_mix_moe_gate_up(void* hid, const void* h, const void* wg, const void* wu, const int32_t* idx, int n, int top, int experts, int ff, int width,
+                         int dtype, void* stream);
+/* y[n] = sum_r wts[n][r] * Wd[idx[n][r]] hid[n*top + r];  Wd [experts][width][ff]. */
+int exl3_mix_moe_down(void* y, const void* hid, const void* wd, const int32_t* idx, const float* wts, int n, int top, int experts, int ff, int width,
+                      int dtype, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif
