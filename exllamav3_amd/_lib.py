@@ -302,6 +302,7 @@ def _declare_mix(l):
     sig("exl3_mix_attn_prefill", vp, vp, i64, vp, i64, vp, vp, i64, vp, vp, vp, vp, i32, i32, i32, i32, i32, f32, i32, i32, vp)
     sig("exl3_mix_attn_decode", vp, vp, i64, vp, vp, vp, i64, vp, vp, vp, i32, i32, i32, i32, i32, f32, i32, i32, vp)
     sig("exl3_mix_gla_scan", vp, vp, vp, i64, vp, i64, vp, i64, vp, i64, vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, f32, f32, i32, vp)
+    sig("exl3_mix_gla_segmented", vp, vp, vp, i64, vp, i64, vp, i64, vp, i64, vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, f32, f32, i32, i32, vp, vp, i32, vp)
     sig("exl3_mix_gla_out", vp, vp, vp, vp, i64, f32, i32, i32, i32, i32, vp)
     sig("exl3_mix_topk_softmax", vp, vp, vp, i32, i32, i32, vp)
     sig("exl3_mix_moe_gate_up", vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, vp)

@@ -125,7 +125,8 @@ def attn_decode(out, q_view, ring_k, ring_v, gate_view, sink, slots, len_after, 
                                                n, heads, kv_heads, dim, vdim, scale, window, code(out.dtype), _stream(out)))
 
 
-def gla_scan(o, state, q_view, k_view, v_view, lr_view, a2, a2_bias, cu, slots, pos0, tau: float, q_scale: float, chunked: bool = False):
+def gla_scan(o, state, q_view, k_view, v_view, lr_view, a2, a2_bias, cu, slots, pos0, tau: float, q_scale: float, segments: tuple[int, int] | None = None):
+    """segments = (segs, seg_len): the time axis of every sequence cut into parallel segments (long prompts); None: one workgroup chain per sequence."""
     n, heads, vdim = o.shape
     n_slots, h2, dim, v2 = state.shape
     rank = a2.shape[1]
@@ -135,10 +136,16 @@ def gla_scan(o, state, q_view, k_view, v_view, lr_view, a2, a2_bias, cu, slots, 
         _f32c(a2_bias, "a2_bias")
     batch = slots.numel()
     _req(cu.numel() == batch + 1 and pos0.numel() == batch, "gla_scan: batch tensors")
-    fn = _lib.mixlib().exl3_mix_gla_chunked if chunked else _lib.mixlib().exl3_mix_gla_scan
-    _check(fn(_p(o), _p(state), _p(q_view), _view(q_view, heads * dim, "q"), _p(k_view), _view(k_view, heads * dim, "k"), _p(v_view),
-              _view(v_view, heads * vdim, "v"), _p(lr_view), _view(lr_view, rank, "lr"), _p(a2), _p(a2_bias), _p(cu), _p(slots), _p(pos0),
-              batch, heads, dim, vdim, rank, tau, q_scale, code(q_view.dtype), _stream(o)))
+    args = (_p(o), _p(state), _p(q_view), _view(q_view, heads * dim, "q"), _p(k_view), _view(k_view, heads * dim, "k"), _p(v_view),
+            _view(v_view, heads * vdim, "v"), _p(lr_view), _view(lr_view, rank, "lr"), _p(a2), _p(a2_bias), _p(cu), _p(slots), _p(pos0),
+            batch, heads, dim, vdim, rank, tau, q_scale)
+    if segments is None:
+        _check(_lib.mixlib().exl3_mix_gla_scan(*args, code(q_view.dtype), _stream(o)))
+        return
+    segs, seg_len = segments
+    seg_state = torch.empty((batch * segs, heads, dim, vdim), dtype=torch.float32, device=o.device)
+    seg_decay = torch.empty((batch * segs, heads, dim), dtype=torch.float32, device=o.device)
+    _check(_lib.mixlib().exl3_mix_gla_segmented(*args, segs, seg_len, _p(seg_state), _p(seg_decay), code(q_view.dtype), _stream(o)))
 
 
 def gla_out(out, o, w, g_view, eps: float):

@@ -93,13 +93,13 @@ class SlidingSinkAttention:
 
 
 class GatedLinearAttention:
-    # rows of a prompt step from which the chunked matrix-core kernel takes over from the token-by-token scan
-    CHUNKED_MIN_ROWS = 64
+    # prompt steps whose longest sequence has at least this many rows are cut into parallel time segments (mix_ops.gla_scan)
+    SEGMENT_MIN_ROWS = 256
+    SEGMENT_TARGET_WORKGROUPS = 1024
 
     def __init__(self, width: int, heads: int, dim: int, vdim: int, tau: float, eps: float):
         self.width, self.heads, self.dim, self.vdim, self.tau, self.eps = width, heads, dim, vdim, float(tau), float(eps)
         self.q_scale = float(dim) ** -0.5
-        self.use_chunked = True
 
     def load(self, stc, prefix: str, dtype, device, extra_parts=()):
         parts = [(nm, _w(stc, prefix + nm, dtype, device), None) for nm in ("q", "k", "v", "g", "a1")]
@@ -115,11 +115,23 @@ class GatedLinearAttention:
     def state_specs(self) -> list[StateSpec]:
         return [StateSpec("S", (self.heads, self.dim, self.vdim), torch.float32)]
 
+    def segments(self, sb: StepBatch) -> tuple[int, int] | None:
+        """(segments per sequence, rows per segment) for a long prompt step: enough workgroups to fill the device, segments of at least 64 rows."""
+        if sb.max_rows < self.SEGMENT_MIN_ROWS:
+            return None
+        chains = sb.batch * self.heads * ((self.vdim + 63) // 64)
+        segs = min(max(1, -(-self.SEGMENT_TARGET_WORKGROUPS // chains)), sb.max_rows // 64)
+        if segs < 2:
+            return None
+        seg_len = -(-sb.max_rows // segs)
+        seg_len = -(-seg_len // 16) * 16
+        return -(-sb.max_rows // seg_len), seg_len
+
     def forward(self, h: torch.Tensor, sb: StepBatch, state: dict) -> tuple[torch.Tensor, dict]:
         p = self.inp(h)
         o = torch.empty((sb.n, self.heads, self.vdim), dtype=torch.float32, device=h.device)
-        chunked = self.use_chunked and hasattr(mix_ops._lib.mixlib(), "exl3_mix_gla_chunked") and sb.max_rows >= self.CHUNKED_MIN_ROWS
-        mix_ops.gla_scan(o, state["S"], p["q"], p["k"], p["v"], p["a1"], self.a2, self.a2_bias, sb.cu, sb.slots, sb.pos0, self.tau, self.q_scale, chunked=chunked)
+        mix_ops.gla_scan(o, state["S"], p["q"], p["k"], p["v"], p["a1"], self.a2, self.a2_bias, sb.cu, sb.slots, sb.pos0, self.tau, self.q_scale,
+                         segments=self.segments(sb))
         out = torch.empty((sb.n, self.heads * self.vdim), dtype=self.dtype, device=h.device)
         mix_ops.gla_out(out, o, self.norm_w, p["g"], self.eps)
         return F.linear(out, self.w_o), p

@@ -83,6 +83,15 @@ int exl3_mix_gla_scan(float* o, float* state, const void* q, int64_t q_ld, const
                       const void* lr, int64_t lr_ld, const void* a2, const float* a2_bias, const int32_t* cu, const int32_t* slots, const int32_t* pos0,
                       int batch, int heads, int dim, int vdim, int rank, float tau, float q_scale, int dtype, void* stream);
 
+/* The same results (up to float32 rounding) for long prompts, with the time axis cut into `segs` segments of `seg_len` rows per sequence
+ * (segs * seg_len >= the longest sequence of the step) that run in parallel: every segment first runs from a zero state and leaves its local
+ * state and the product of its decays, a short pass chains these into the state each segment starts from (and the slot's final state), and
+ * every segment runs again from there and writes its outputs.  seg_state [batch*segs][heads][dim][vdim], seg_decay [batch*segs][heads][dim]: scratch. */
+int exl3_mix_gla_segmented(float* o, float* state, const void* q, int64_t q_ld, const void* k, int64_t k_ld, const void* v, int64_t v_ld,
+                           const void* lr, int64_t lr_ld, const void* a2, const float* a2_bias, const int32_t* cu, const int32_t* slots, const int32_t* pos0,
+                           int batch, int heads, int dim, int vdim, int rank, float tau, float q_scale, int segs, int seg_len,
+                           float* seg_state, float* seg_decay, int dtype, void* stream);
+
 /* out[n][h*vdim + v] = o[n][h][v] / sqrt(mean_v(o[n][h]^2) + eps) * w[v] * silu(g[n][h*vdim + v]) */
 int exl3_mix_gla_out(void* out, const float* o, const float* w, const void* g, int64_t g_ld, float eps, int n, int heads, int vdim, int dtype, void* stream);
 
