@@ -1,5 +1,6 @@
-// Unquantized experts for a few rows (decode, short prompts, and the float32 path): one wave per output element streams the chosen
-// expert's weight row.  Sums are float32.  Long bfloat16 prompts go through the grouped matrix-core kernel instead (mix_moe_mfma.hip).
+// Unquantized experts.  A few rows (decode, short prompts): one wave per output element streams the chosen expert's weight row, sums in
+// float32.  Many rows (prompts): the host sorts the rows by expert and runs one vendor matrix product per expert and projection; the
+// activation between them and the weighted un-sort are the two small kernels at the end of this file.
 #include "mix_common.cuh"
 
 template <typename T>
@@ -42,6 +43,44 @@ __global__ __launch_bounds__(256) void moe_down_kernel(T* __restrict__ y, const 
         acc += wts[(int64_t) n * top + r] * wave_sum(a);
     }
     if (lane == 0) y[(int64_t) n * width + col] = from_f<T>(acc);
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void silu_mul_kernel(T* __restrict__ out, const T* __restrict__ g, const T* __restrict__ u, int64_t count)
+{
+    for (int64_t i = (int64_t) blockIdx.x * 256 + threadIdx.x; i < count; i += (int64_t) gridDim.x * 256)
+        out[i] = from_f<T>(silu_f(to_f(g[i])) * to_f(u[i]));
+}
+
+// y[n] = sum_r wts[n][r] * sorted[where[n*top + r]]: the rows of the expert-sorted result back in token order, weighted.
+template <typename T>
+__global__ __launch_bounds__(256) void moe_combine_kernel(T* __restrict__ y, const T* __restrict__ sorted, const int32_t* __restrict__ where,
+                                                          const float* __restrict__ wts, int top, int width)
+{
+    const int n = blockIdx.x;
+    for (int c = threadIdx.x; c < width; c += 256)
+    {
+        float acc = 0.f;
+        for (int r = 0; r < top; ++r) acc += wts[(int64_t) n * top + r] * to_f(sorted[(int64_t) where[(int64_t) n * top + r] * width + c]);
+        y[(int64_t) n * width + c] = from_f<T>(acc);
+    }
+}
+
+extern "C" int exl3_mix_silu_mul(void* out, const void* g, const void* u, int64_t count, int dtype, void* stream)
+{
+    MIX_CHECK(out && g && u && count >= 0, "mix_silu_mul: bad arguments");
+    if (count == 0) return EXL3_MIX_OK;
+    const int blocks = (int) ((count + 255) / 256 > 8192 ? 8192 : (count + 255) / 256);
+    MIX_DISPATCH_T(dtype, hipLaunchKernelGGL(silu_mul_kernel<T>, dim3(blocks), dim3(256), 0, (hipStream_t) stream, (T*) out, (const T*) g, (const T*) u, count));
+    return mix_check_launch("mix_silu_mul");
+}
+
+extern "C" int exl3_mix_moe_combine(void* y, const void* sorted, const int32_t* where, const float* wts, int n, int top, int width, int dtype, void* stream)
+{
+    MIX_CHECK(y && sorted && where && wts && n >= 0 && top > 0 && width > 0, "mix_moe_combine: bad arguments");
+    if (n == 0) return EXL3_MIX_OK;
+    MIX_DISPATCH_T(dtype, hipLaunchKernelGGL(moe_combine_kernel<T>, dim3(n), dim3(256), 0, (hipStream_t) stream, (T*) y, (const T*) sorted, where, wts, top, width));
+    return mix_check_launch("mix_moe_combine");
 }
 
 extern "C" int exl3_mix_moe_gate_up(void* hid, const void* h, const void* wg, const void* wu, const int32_t* idx, int n, int top, int experts, int ff, int width,

@@ -101,12 +101,25 @@ def attn_store(v_norm, ring_k, ring_v, k_view, v_view, tok_seq, tok_pos, slots, 
                                               code(v_norm.dtype), _stream(v_norm)))
 
 
-def attn_prefill(out, q_view, k_view, v_norm, gate_view, sink, cu, tok_seq, tok_pos, heads: int, scale: float, window: int):
+# prompt steps from this many rows on (bfloat16, head sizes <= 256) run on the matrix cores
+ATTN_MFMA_MIN_ROWS = 32
+
+
+def attn_prefill(out, q_view, k_view, v_norm, gate_view, sink, cu, tok_seq, tok_pos, heads: int, scale: float, window: int, max_rows: int = 0, mfma: bool | None = None):
+    """max_rows: the longest sequence of the step (host number; needed for the matrix-core kernel's grid).  mfma None: chosen by size and type."""
     n, kv_heads, vdim = v_norm.shape
     dim = q_view.shape[1] // heads
     _req(out.is_contiguous() and out.shape == (n, heads * vdim) and out.dtype == q_view.dtype == k_view.dtype == v_norm.dtype, "attn_prefill: out / types")
     if sink is not None:
         _f32c(sink, "sink"); _req(sink.numel() == heads, "attn_prefill: sink")
+    if mfma is None:
+        mfma = out.dtype == torch.bfloat16 and max_rows >= ATTN_MFMA_MIN_ROWS and dim <= 256 and vdim <= 256
+    if mfma:
+        _req(out.dtype == torch.bfloat16 and max_rows > 0 and v_norm.is_contiguous(), "attn_prefill: the matrix-core kernel takes bfloat16 and the step's longest sequence")
+        _check(_lib.mixlib().exl3_mix_attn_prefill_mfma(_p(out), _p(q_view), _view(q_view, heads * dim, "q"), _p(k_view), _view(k_view, kv_heads * dim, "k"), _p(v_norm),
+                                                         _p(gate_view), 0 if gate_view is None else _view(gate_view, heads, "gate"), _p(sink), _p(cu),
+                                                         cu.numel() - 1, max_rows, heads, kv_heads, dim, vdim, scale, window, _stream(out)))
+        return
     _check(_lib.mixlib().exl3_mix_attn_prefill(_p(out), _p(q_view), _view(q_view, heads * dim, "q"), _p(k_view), _view(k_view, kv_heads * dim, "k"), _p(v_norm),
                                                 _p(gate_view), 0 if gate_view is None else _view(gate_view, heads, "gate"), _p(sink), _p(cu), _p(tok_seq), _p(tok_pos),
                                                 n, heads, kv_heads, dim, vdim, scale, window, code(out.dtype), _stream(out)))
@@ -181,3 +194,29 @@ def moe_down(y, hid, wd, idx, wts):
          "moe_down: shapes")
     _i32c(idx, "idx"); _f32c(wts, "wts")
     _check(_lib.mixlib().exl3_mix_moe_down(_p(y), _p(hid), _p(wd), _p(idx), _p(wts), n, top, experts, ff, width, code(y.dtype), _stream(y)))
+
+
+def moe_grouped(y, h, wg, wu, wd, idx, wts):
+    """Experts of many rows: rows sorted by expert (device), one host read of the per-expert counts, then per expert three vendor matrix products
+    with the activation kernel between them, and the weighted un-sort.  Same result as moe_gate_up + moe_down up to rounding."""
+    n, width = h.shape
+    experts, ff, _ = wg.shape
+    top = idx.shape[1]
+    flat = idx.reshape(-1).long()
+    order = torch.sort(flat, stable=True).indices
+    counts = torch.zeros(experts, dtype=torch.int32, device=h.device).index_add_(0, flat, torch.ones_like(flat, dtype=torch.int32)).tolist()
+    where = torch.empty(n * top, dtype=torch.int32, device=h.device)
+    where[order] = torch.arange(n * top, dtype=torch.int32, device=h.device)
+    xs = h.index_select(0, order // top)
+    out = torch.empty((n * top, width), dtype=h.dtype, device=h.device)
+    hid = torch.empty((n * top, ff), dtype=h.dtype, device=h.device)
+    lib, at = _lib.mixlib(), 0
+    for e, c in enumerate(counts):
+        if c == 0:
+            continue
+        seg = xs[at: at + c]
+        g, u = torch.nn.functional.linear(seg, wg[e]), torch.nn.functional.linear(seg, wu[e])
+        _check(lib.exl3_mix_silu_mul(_p(hid[at: at + c]), _p(g), _p(u), c * ff, code(h.dtype), _stream(h)))
+        torch.mm(hid[at: at + c], wd[e].t(), out=out[at: at + c])
+        at += c
+    _check(lib.exl3_mix_moe_combine(_p(y), _p(out), _p(where), _p(wts), n, top, width, code(h.dtype), _stream(h)))

@@ -88,7 +88,8 @@ class SlidingSinkAttention:
         if sb.decode:
             mix_ops.attn_decode(out, p["q"], state["ring_k"], state["ring_v"], p.get("g"), self.sink, sb.slots, sb.len_after, self.heads, self.scale)
         else:
-            mix_ops.attn_prefill(out, p["q"], p["k"], v_norm, p.get("g"), self.sink, sb.cu, sb.tok_seq, sb.tok_pos, self.heads, self.scale, self.window)
+            mix_ops.attn_prefill(out, p["q"], p["k"], v_norm, p.get("g"), self.sink, sb.cu, sb.tok_seq, sb.tok_pos, self.heads, self.scale, self.window,
+                                 max_rows=sb.max_rows)
         return F.linear(out, self.w_o), p
 
 
@@ -156,8 +157,8 @@ class PolyNormMLP:
 
 
 class SparseExperts:
-    # rows from which the grouped matrix-core kernels take over from the weight-streaming ones (bfloat16 only)
-    GROUPED_MIN_ROWS = 32
+    # rows from which the expert-sorted matrix products take over from the weight-streaming kernels
+    GROUPED_MIN_ROWS = 64
 
     def __init__(self, width: int, ff: int, experts: int, top: int):
         if not 0 < top <= experts:
@@ -180,7 +181,7 @@ class SparseExperts:
         wts = torch.empty((sb.n, self.top), dtype=torch.float32, device=h.device)
         mix_ops.topk_softmax(idx, wts, logits)
         y = torch.empty((sb.n, self.width), dtype=self.dtype, device=h.device)
-        if self.dtype == torch.bfloat16 and sb.n >= self.GROUPED_MIN_ROWS and hasattr(mix_ops, "moe_grouped"):
+        if sb.n >= self.GROUPED_MIN_ROWS:
             mix_ops.moe_grouped(y, h, self.w_gate, self.w_up, self.w_down, idx, wts)
         else:
             hid = torch.empty((sb.n * self.top, self.ff), dtype=self.dtype, device=h.device)

@@ -68,6 +68,12 @@ int exl3_mix_attn_prefill(void* out, const void* q, int64_t q_ld, const void* k,
                           const void* gate, int64_t gate_ld, const float* sink, const int32_t* cu, const int32_t* tok_seq, const int32_t* tok_pos,
                           int n, int heads, int kv_heads, int dim, int vdim, float scale, int window, int dtype, void* stream);
 
+/* The same on the matrix cores, bfloat16 only (scores, maxima, exponentials and sums stay float32; the weights are rounded to bfloat16 for the
+ * product with the values): dim, vdim <= 256; `max_rows` = the longest sequence of the step. */
+int exl3_mix_attn_prefill_mfma(void* out, const void* q, int64_t q_ld, const void* k, int64_t k_ld, const void* v_norm,
+                               const void* gate, int64_t gate_ld, const float* sink, const int32_t* cu,
+                               int batch, int max_rows, int heads, int kv_heads, int dim, int vdim, float scale, int window, void* stream);
+
 /* The same for one new row per sequence against the ring buffers (which already hold the row's own key and value):
  * row b sees the min(len_after[b], window) newest entries of slot slots[b]. */
 int exl3_mix_attn_decode(void* out, const void* q, int64_t q_ld, const void* ring_k, const void* ring_v,
@@ -105,6 +111,11 @@ int exl3_mix_moe_gate_up(void* hid, const void* h, const void* wg, const void* w
 /* y[n] = sum_r wts[n][r] * Wd[idx[n][r]] hid[n*top + r];  Wd [experts][width][ff]. */
 int exl3_mix_moe_down(void* y, const void* hid, const void* wd, const int32_t* idx, const float* wts, int n, int top, int experts, int ff, int width,
                       int dtype, void* stream);
+
+/* Experts of many rows run as vendor matrix products over rows sorted by expert; these two kernels sit between and behind them:
+ * out = silu(g) * u element by element, and y[n] = sum_r wts[n][r] * sorted[where[n*top + r]] (rows back in token order, weighted). */
+int exl3_mix_silu_mul(void* out, const void* g, const void* u, int64_t count, int dtype, void* stream);
+int exl3_mix_moe_combine(void* y, const void* sorted, const int32_t* where, const float* wts, int n, int top, int width, int dtype, void* stream);
 
 #ifdef __cplusplus
 }

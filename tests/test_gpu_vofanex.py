@@ -45,7 +45,7 @@ TOL = {torch.float32: 2e-5, torch.bfloat16: 3e-2}
 # ---- mechanisms alone -------------------------------------------------------------------------------------------------------
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("H,G,d,dv,W,lens", [(4, 2, 16, 24, 5, [17, 1, 9]), (3, 3, 40, 72, 64, [70]), (2, 1, 8, 8, 1, [6, 3]), (6, 2, 32, 130, 7, [20])])
+@pytest.mark.parametrize("H,G,d,dv,W,lens", [(4, 2, 16, 24, 5, [17, 1, 9]), (3, 3, 40, 72, 64, [70]), (2, 1, 8, 8, 1, [6, 3]), (6, 2, 32, 130, 7, [20]), (2, 1, 96, 96, 37, [150, 66]), (1, 1, 136, 64, 100, [131])])
 def test_attention_prefill_then_decode_matches_oracle(gpu, dtype, H, G, d, dv, W, lens):
     from exllamav3_amd import mix_ops
     g = torch.Generator().manual_seed(H * 100 + W)
@@ -68,9 +68,11 @@ def test_attention_prefill_then_decode_matches_oracle(gpu, dtype, H, G, d, dv, W
     vn = torch.empty((n, G, dv), dtype=dtype, device=gpu)
     mix_ops.attn_store(vn, ring_k, ring_v, k, v, seq, pos, sl, la, 1e-5)
     out = torch.empty((n, H * dv), dtype=dtype, device=gpu)
-    mix_ops.attn_prefill(out, q, k, vn, gt, sink.to(gpu), cu, seq, pos, H, scale, W)
     want = torch.cat([r[:l] for r, l in zip(ref, lens)]).flatten(1)
-    assert rel(out, want) < TOL[dtype]
+    for mfma in ([False, True] if dtype == torch.bfloat16 else [False]):           # the lane-per-key kernel and the matrix-core kernel
+        out.fill_(float("nan"))
+        mix_ops.attn_prefill(out, q, k, vn, gt, sink.to(gpu), cu, seq, pos, H, scale, W, max_rows=max(lens), mfma=mfma)
+        assert rel(out, want) < TOL[dtype], f"mfma={mfma}"
     # decode steps, all sequences together
     for s in range(extra):
         cur = [l + s for l in lens]
@@ -220,7 +222,7 @@ def test_router_and_experts_match_oracle(gpu, dtype, n, E, top, ff, width):
     mix_ops.moe_gate_up(hid, h.to(gpu), wg.to(gpu), wu.to(gpu), idx)
     mix_ops.moe_down(y, hid, wd.to(gpu), idx, wts)
     assert rel(y, ref) < TOL[dtype]
-    if dtype == torch.bfloat16 and hasattr(mix_ops, "moe_grouped"):
+    if True:
         y2 = torch.empty_like(y)
         mix_ops.moe_grouped(y2, h.to(gpu), wg.to(gpu), wu.to(gpu), wd.to(gpu), idx, wts)
         assert rel(y2, ref) < TOL[dtype]
