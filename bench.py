@@ -53,6 +53,9 @@ def parse():
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-extra", action="store_true", help="skip the other BASELINE configs (1B bs 1, 8B bs 16, 8B bs 1 with attention) on the JSON line")
     ap.add_argument("--prefill-tokens", type=int, default=4096)
+    ap.add_argument("--mixer-family", action="store_true",
+                    help="instead of the default workload: layer times of the unquantized mixer family (Vofanex) beside the EXL3 Llama layer of equal size, and its kernels' rooflines")
+    ap.add_argument("--mixer-sizes", default="", help="with --mixer-family: comma-separated sizes (1b, 8b; default both)")
     ap.add_argument("--variant", type=int, default=1)
     ap.add_argument("--attention", action="store_true", help="include decode attention over the quantized KV cache (context = 1000 tokens) in the timed step")
     ap.add_argument("--unfused", action="store_true", help="one launch per reference op instead of the fused pipeline")
@@ -248,6 +251,9 @@ def pinned_logits_check(model_name, K, cb, bsz, dev, pipeline, tol=3e-2, ctx=Non
 
 def main():
     args = parse()
+    if args.mixer_family:
+        from exllamav3_amd import mixer_bench
+        sys.exit(mixer_bench.run(args))
     import torch
     from exllamav3_amd import ext
     from exllamav3_amd.llama_path import SHAPES, SyntheticEXL3Llama

@@ -1,6 +1,6 @@
 // Sliding-window attention with a learned sink and a head-wise output gate: cache store (value norm, ring buffers) and the exact
-// float32 form of prefill and decode -- one wave per (row, query head), keys of the window across the lanes, an online softmax that
-// starts from the sink.  The matrix-core prefill kernel for bfloat16 lives in mix_attn_mfma.hip; this file is the float32 path and
+// float32 form of prefill and decode -- one workgroup per (row, query head), keys of the window across lanes and waves, an online softmax
+// that starts from the sink.  The matrix-core prefill kernel for bfloat16 lives in mix_attn_mfma.hip; this file is the float32 path and
 // the decode path of both element types.
 #include "mix_common.cuh"
 
@@ -35,20 +35,34 @@ __global__ __launch_bounds__(64) void attn_store_kernel(T* __restrict__ v_norm, 
     }
 }
 
-// One wave per (row, head).  Keys kb + j * k_step, values vb + j * v_step, j < count.  MAXV = ceil(vdim / 64) accumulators per lane.
+// One workgroup of AT_WAVES waves per (row, query head).  Keys kb + j * k_step, values vb + j * v_step, j < count: wave w takes the 64-key chunks
+// w, w + AT_WAVES, ... (one key per lane, its row read in 16-byte pieces when the layout allows), keeps its own running maximum, sum and
+// value accumulators (MAXV = ceil(vdim / 64) per lane), and the waves are merged through LDS at the end.  Wave 0 starts from the sink.
+#define AT_WAVES 4
+
+template <typename T> struct kvec;
+template <> struct kvec<bf16_t> { static constexpr int N = 8; };
+template <> struct kvec<float> { static constexpr int N = 4; };
+
 template <typename T, int MAXV>
 __device__ __forceinline__ void attn_row(T* __restrict__ out, const T* __restrict__ q, const T* __restrict__ kb, int64_t k_step, const T* __restrict__ vb,
-                                         int64_t v_step, int count, int dim, int vdim, float scale, bool has_sink, float sink, float gate,
-                                         float* qs, float* ps)
+                                         int64_t v_step, int count, int dim, int vdim, float scale, bool has_sink, float sink, float gate, bool k_vec,
+                                         float* smem)
 {
-    const int lane = threadIdx.x;
-    for (int i = lane; i < dim; i += 64) qs[i] = to_f(q[i]);
+    float* qs = smem;                                   // [dim]
+    float* ps = qs + dim;                               // [AT_WAVES][64]
+    float* mg = ps + AT_WAVES * 64;                     // [AT_WAVES][2 + MAXV * 64]: m, l, accumulators
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    for (int i = threadIdx.x; i < dim; i += 64 * AT_WAVES) qs[i] = to_f(q[i]);
     __syncthreads();
-    float m = has_sink ? sink : -INFINITY, l = has_sink ? 1.0f : 0.0f;
+    const bool seeded = has_sink && w == 0;
+    float m = seeded ? sink : -INFINITY, l = seeded ? 1.0f : 0.0f;
     float acc[MAXV];
     #pragma unroll
     for (int i = 0; i < MAXV; ++i) acc[i] = 0.f;
-    for (int j0 = 0; j0 < count; j0 += 64)
+    float* pw = ps + w * 64;
+    constexpr int VN = kvec<T>::N;
+    for (int j0 = w * 64; j0 < count; j0 += 64 * AT_WAVES)
     {
         const int j = j0 + lane;
         float s = -INFINITY;
@@ -56,17 +70,27 @@ __device__ __forceinline__ void attn_row(T* __restrict__ out, const T* __restric
         {
             const T* kr = kb + (int64_t) j * k_step;
             float d = 0.f;
-            for (int c = 0; c < dim; ++c) d += qs[c] * to_f(kr[c]);
+            if (k_vec)
+            {
+                for (int c = 0; c < dim; c += VN)
+                {
+                    union { uint4 v; T e[VN]; } t;
+                    t.v = *(const uint4*) (kr + c);
+                    #pragma unroll
+                    for (int e = 0; e < VN; ++e) d += qs[c + e] * to_f(t.e[e]);
+                }
+            }
+            else
+                for (int c = 0; c < dim; ++c) d += qs[c] * to_f(kr[c]);
             s = d * scale;
         }
         const float m_new = fmaxf(m, wave_max(s));          // finite: j0 < count, so lane 0 of the chunk holds a score
         const float p = (j < count) ? expf(s - m_new) : 0.f;
-        const float corr = expf(m - m_new);                 // m = -inf (no sink, first chunk): 0
+        const float corr = expf(m - m_new);                 // m = -inf (nothing yet): 0
         l = l * corr + wave_sum(p);
         m = m_new;
-        __syncthreads();
-        ps[lane] = p;
-        __syncthreads();
+        pw[lane] = p;
+        __builtin_amdgcn_wave_barrier();                    // LDS serves a wave's accesses in order: its own stores are visible to the reads below
         const int cnt = min(64, count - j0);
         #pragma unroll
         for (int i = 0; i < MAXV; ++i)
@@ -74,11 +98,34 @@ __device__ __forceinline__ void attn_row(T* __restrict__ out, const T* __restric
             const int c = lane + 64 * i;
             float a = acc[i] * corr;
             if (c < vdim)
-                for (int jj = 0; jj < cnt; ++jj) a += ps[jj] * to_f(vb[(int64_t) (j0 + jj) * v_step + c]);
+                for (int jj = 0; jj < cnt; ++jj) a += pw[jj] * to_f(vb[(int64_t) (j0 + jj) * v_step + c]);
             acc[i] = a;
         }
+        __builtin_amdgcn_wave_barrier();
     }
-    const float f = (l > 0.f ? 1.0f / l : 0.f) * gate;
+    // merge the waves: wave 0 rescales every wave's partial to the common maximum
+    float* mine = mg + w * (2 + MAXV * 64);
+    if (lane == 0) { mine[0] = m; mine[1] = l; }
+    #pragma unroll
+    for (int i = 0; i < MAXV; ++i) mine[2 + i * 64 + lane] = acc[i];
+    __syncthreads();
+    if (w != 0) return;
+    float mt = -INFINITY;
+    #pragma unroll
+    for (int ww = 0; ww < AT_WAVES; ++ww) mt = fmaxf(mt, mg[ww * (2 + MAXV * 64)]);
+    float lt = 0.f;
+    #pragma unroll
+    for (int i = 0; i < MAXV; ++i) acc[i] = 0.f;
+    #pragma unroll
+    for (int ww = 0; ww < AT_WAVES; ++ww)
+    {
+        const float* o = mg + ww * (2 + MAXV * 64);
+        const float f = (o[0] == -INFINITY) ? 0.f : expf(o[0] - mt);
+        lt += o[1] * f;
+        #pragma unroll
+        for (int i = 0; i < MAXV; ++i) acc[i] += o[2 + i * 64 + lane] * f;
+    }
+    const float f = (lt > 0.f ? 1.0f / lt : 0.f) * gate;
     #pragma unroll
     for (int i = 0; i < MAXV; ++i)
     {
@@ -87,42 +134,47 @@ __device__ __forceinline__ void attn_row(T* __restrict__ out, const T* __restric
     }
 }
 
+template <typename T>
+__device__ __forceinline__ bool rows_are_16_byte(const T* base, int64_t step, int dim)
+{
+    return ((uintptr_t) base % 16 == 0) && ((step * (int64_t) sizeof(T)) % 16 == 0) && (dim % kvec<T>::N == 0);
+}
+
 template <typename T, int MAXV>
-__global__ __launch_bounds__(64) void attn_prefill_kernel(T* __restrict__ out, const T* __restrict__ q, int64_t q_ld, const T* __restrict__ k, int64_t k_ld,
+__global__ __launch_bounds__(64 * AT_WAVES) void attn_prefill_kernel(T* __restrict__ out, const T* __restrict__ q, int64_t q_ld, const T* __restrict__ k, int64_t k_ld,
                                                           const T* __restrict__ v_norm, const T* __restrict__ gate, int64_t gate_ld, const float* __restrict__ sink,
                                                           const int32_t* __restrict__ cu, const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ tok_pos,
                                                           int heads, int kv_heads, int dim, int vdim, float scale, int window)
 {
     extern __shared__ float smem[];
-    float* qs = smem; float* ps = smem + dim;
     const int n = blockIdx.x, h = blockIdx.y;
     const int g = h / (heads / kv_heads);
     const int b = tok_seq[n], first = cu[b];
     const int i = n - first;                                  // the row's place in its sequence == its position (the sequence starts in this step)
     const int lo = max(0, i - window + 1);
     const float gt = gate ? sigmoid_f(to_f(gate[(int64_t) n * gate_ld + h])) : 1.0f;
-    attn_row<T, MAXV>(out + ((int64_t) n * heads + h) * vdim, q + (int64_t) n * q_ld + (int64_t) h * dim,
-                      k + (int64_t) (first + lo) * k_ld + (int64_t) g * dim, k_ld,
+    const T* kb = k + (int64_t) (first + lo) * k_ld + (int64_t) g * dim;
+    attn_row<T, MAXV>(out + ((int64_t) n * heads + h) * vdim, q + (int64_t) n * q_ld + (int64_t) h * dim, kb, k_ld,
                       v_norm + ((int64_t) (first + lo) * kv_heads + g) * vdim, (int64_t) kv_heads * vdim,
-                      i - lo + 1, dim, vdim, scale, sink != nullptr, sink ? sink[h] : 0.f, gt, qs, ps);
+                      i - lo + 1, dim, vdim, scale, sink != nullptr, sink ? sink[h] : 0.f, gt, rows_are_16_byte(kb, k_ld, dim), smem);
 }
 
 template <typename T, int MAXV>
-__global__ __launch_bounds__(64) void attn_decode_kernel(T* __restrict__ out, const T* __restrict__ q, int64_t q_ld, const T* __restrict__ ring_k,
+__global__ __launch_bounds__(64 * AT_WAVES) void attn_decode_kernel(T* __restrict__ out, const T* __restrict__ q, int64_t q_ld, const T* __restrict__ ring_k,
                                                          const T* __restrict__ ring_v, const T* __restrict__ gate, int64_t gate_ld, const float* __restrict__ sink,
                                                          const int32_t* __restrict__ slots, const int32_t* __restrict__ len_after,
                                                          int heads, int kv_heads, int dim, int vdim, float scale, int window)
 {
     extern __shared__ float smem[];
-    float* qs = smem; float* ps = smem + dim;
     const int n = blockIdx.x, h = blockIdx.y;
     const int g = h / (heads / kv_heads);
     const int count = min(len_after[n], window);
     const int64_t base = (int64_t) slots[n] * window * kv_heads + g;
     const float gt = gate ? sigmoid_f(to_f(gate[(int64_t) n * gate_ld + h])) : 1.0f;
+    const T* kb = ring_k + base * dim;
     attn_row<T, MAXV>(out + ((int64_t) n * heads + h) * vdim, q + (int64_t) n * q_ld + (int64_t) h * dim,
-                      ring_k + base * dim, (int64_t) kv_heads * dim, ring_v + base * vdim, (int64_t) kv_heads * vdim,
-                      count, dim, vdim, scale, sink != nullptr, sink ? sink[h] : 0.f, gt, qs, ps);
+                      kb, (int64_t) kv_heads * dim, ring_v + base * vdim, (int64_t) kv_heads * vdim,
+                      count, dim, vdim, scale, sink != nullptr, sink ? sink[h] : 0.f, gt, rows_are_16_byte(kb, (int64_t) kv_heads * dim, dim), smem);
 }
 
 extern "C" int exl3_mix_attn_store(void* v_norm, void* ring_k, void* ring_v, const void* k, int64_t k_ld, const void* v, int64_t v_ld,
@@ -140,13 +192,14 @@ extern "C" int exl3_mix_attn_store(void* v_norm, void* ring_k, void* ring_v, con
 
 #define ATTN_LAUNCH(KERNEL, ...) \
     do { \
-        const size_t sm = (size_t) (dim + 64) * sizeof(float); \
         const int mv = (vdim + 63) / 64; \
+        const int mvt = mv == 1 ? 1 : (mv == 2 ? 2 : (mv <= 4 ? 4 : 8)); \
+        const size_t sm = (size_t) (dim + AT_WAVES * 64 + AT_WAVES * (2 + mvt * 64)) * sizeof(float); \
         MIX_DISPATCH_T(dtype, \
-            if (mv == 1)      hipLaunchKernelGGL((KERNEL<T, 1>), dim3(n, heads), dim3(64), sm, (hipStream_t) stream, __VA_ARGS__); \
-            else if (mv == 2) hipLaunchKernelGGL((KERNEL<T, 2>), dim3(n, heads), dim3(64), sm, (hipStream_t) stream, __VA_ARGS__); \
-            else if (mv <= 4) hipLaunchKernelGGL((KERNEL<T, 4>), dim3(n, heads), dim3(64), sm, (hipStream_t) stream, __VA_ARGS__); \
-            else              hipLaunchKernelGGL((KERNEL<T, 8>), dim3(n, heads), dim3(64), sm, (hipStream_t) stream, __VA_ARGS__)); \
+            if (mv == 1)      hipLaunchKernelGGL((KERNEL<T, 1>), dim3(n, heads), dim3(64 * AT_WAVES), sm, (hipStream_t) stream, __VA_ARGS__); \
+            else if (mv == 2) hipLaunchKernelGGL((KERNEL<T, 2>), dim3(n, heads), dim3(64 * AT_WAVES), sm, (hipStream_t) stream, __VA_ARGS__); \
+            else if (mv <= 4) hipLaunchKernelGGL((KERNEL<T, 4>), dim3(n, heads), dim3(64 * AT_WAVES), sm, (hipStream_t) stream, __VA_ARGS__); \
+            else              hipLaunchKernelGGL((KERNEL<T, 8>), dim3(n, heads), dim3(64 * AT_WAVES), sm, (hipStream_t) stream, __VA_ARGS__)); \
     } while (0)
 
 static int attn_check(const char* what, int n, int heads, int kv_heads, int dim, int vdim, int window)

@@ -2,8 +2,8 @@
 // v_mfma_f32_16x16x32_bf16, scores, running maximum, exponentials and sums in float32; the softmax starts from the sink, so the sink is one
 // more term of the denominator and nothing else.
 //
-// One workgroup = 64 query rows of one sequence and one head, 4 waves of 16 rows.  Key tiles of 32 rows are staged in LDS once for the four
-// waves: K as stored, V transposed (so that both are read as 16-byte contraction groups).  MFMA operand lane (g = lane / 16, c = lane % 16)
+// One workgroup = 128 query rows of one sequence and one head, 8 waves of 16 rows.  Key tiles of KT = 64 rows (32 for the largest heads, where
+// 64 would not fit 64 KB of LDS) are staged in LDS once for the eight waves: K as stored, V transposed (so that both are read as 16-byte contraction groups).  MFMA operand lane (g = lane / 16, c = lane % 16)
 // holds row / column c and contraction slots 8g .. 8g+7; result lane (g, c) holds rows 4g .. 4g+3 of column c.  A wave's P tile goes
 // through its own LDS patch from the result layout to the operand layout.  Only the key tiles that intersect the window of the block's
 // rows are visited, and a wave skips the tiles outside its own rows' windows.
@@ -12,13 +12,13 @@
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
-#define AM_ROWS 64
-#define AM_KEYS 32
+#define AM_ROWS 128
+#define AM_THREADS 512
 #define AM_PAD 8
 
 // KD: contraction steps of 32 over the (zero-padded) head dim; NV: 16-column tiles of the (padded) value dim.
-template <int KD, int NV>
-__global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ q, int64_t q_ld, const bf16_t* __restrict__ k,
+template <int KD, int NV, int AM_KEYS>
+__global__ __launch_bounds__(AM_THREADS) void attn_prefill_mfma_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ q, int64_t q_ld, const bf16_t* __restrict__ k,
                                                                 int64_t k_ld, const bf16_t* __restrict__ v_norm, const bf16_t* __restrict__ gate, int64_t gate_ld,
                                                                 const float* __restrict__ sink, const int32_t* __restrict__ cu,
                                                                 int heads, int kv_heads, int dim, int vdim, float scale, int window, int k_vec, int v_vec)
@@ -27,7 +27,7 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(bf16_t* __restri
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     uint16_t* k_lds = (uint16_t*) smem_raw;                       // [AM_KEYS][KS]
     uint16_t* vt_lds = k_lds + AM_KEYS * KS;                      // [NV * 16][VS]   (value column, key)
-    uint16_t* p_lds = vt_lds + NV * 16 * VS;                      // [4 waves][16][PS]
+    uint16_t* p_lds = vt_lds + NV * 16 * VS;                      // [8 waves][16][PS]
 
     const int b = blockIdx.y, h = blockIdx.z;
     const int first = cu[b], len = cu[b + 1] - first;
@@ -69,7 +69,7 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(bf16_t* __restri
     {
         __syncthreads();                                           // the previous tile's operand reads are over
         // stage K [32][DP] (zero beyond dim / len) and V^T [vdim][32]
-        for (int idx = threadIdx.x; idx < AM_KEYS * (DP / 8); idx += 256)
+        for (int idx = threadIdx.x; idx < AM_KEYS * (DP / 8); idx += AM_THREADS)
         {
             const int r = idx / (DP / 8), cg = idx - r * (DP / 8);
             const int j = j0 + r;
@@ -83,7 +83,7 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(bf16_t* __restri
             }
             *(uint4*) (k_lds + r * KS + cg * 8) = t.v;
         }
-        for (int idx = threadIdx.x; idx < AM_KEYS * NV * 2; idx += 256)
+        for (int idx = threadIdx.x; idx < AM_KEYS * NV * 2; idx += AM_THREADS)
         {
             const int cg = idx / AM_KEYS, r = idx - cg * AM_KEYS;               // consecutive lanes: consecutive keys of one column group (LDS stores side by side)
             const int j = j0 + r;
@@ -103,37 +103,51 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(bf16_t* __restri
         const bool skip = !wave_live || j0 > wq_hi || j0 + AM_KEYS - 1 < wq_lo - window + 1;
         if (!skip)
         {
-            f32x4 s0 = f32x4{0.f, 0.f, 0.f, 0.f}, s1 = s0;
+            constexpr int NS = AM_KEYS / 16;                                   // 16-key score tiles
+            f32x4 sc[NS];
+            #pragma unroll
+            for (int u = 0; u < NS; ++u) sc[u] = f32x4{0.f, 0.f, 0.f, 0.f};
             #pragma unroll
             for (int s = 0; s < KD; ++s)
             {
-                const bf16x8 k0 = *(const bf16x8*) (k_lds + c * KS + s * 32 + g * 8);
-                const bf16x8 k1 = *(const bf16x8*) (k_lds + (16 + c) * KS + s * 32 + g * 8);
-                s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[s], k0, s0, 0, 0, 0);
-                s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[s], k1, s1, 0, 0, 0);
+                #pragma unroll
+                for (int u = 0; u < NS; ++u)
+                {
+                    const bf16x8 kf = *(const bf16x8*) (k_lds + (u * 16 + c) * KS + s * 32 + g * 8);
+                    sc[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[s], kf, sc[u], 0, 0, 0);
+                }
             }
             float corr[4];
             #pragma unroll
             for (int i = 0; i < 4; ++i)
             {
                 const int qi = q0 + w * 16 + g * 4 + i;                       // this result row's position
-                const int ja = j0 + c, jb = j0 + 16 + c;
-                const bool oka = ja <= qi && qi - ja < window && qi < len;
-                const bool okb = jb <= qi && qi - jb < window && qi < len;
-                const float a = oka ? s0[i] * scale : -INFINITY, bb = okb ? s1[i] * scale : -INFINITY;
-                float mx = fmaxf(a, bb);
+                float sv[NS];
+                float mx = -INFINITY;
+                #pragma unroll
+                for (int u = 0; u < NS; ++u)
+                {
+                    const int j = j0 + u * 16 + c;
+                    const bool ok = j <= qi && qi - j < window && qi < len;
+                    sv[u] = ok ? sc[u][i] * scale : -INFINITY;
+                    mx = fmaxf(mx, sv[u]);
+                }
                 #pragma unroll
                 for (int o = 8; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
                 const float mn = fmaxf(m[i], mx);                              // finite: m starts at the sink or at -1e30
-                const float pa = oka ? expf(a - mn) : 0.f, pb = okb ? expf(bb - mn) : 0.f;
-                float sum = pa + pb;
+                float sum = 0.f;
+                #pragma unroll
+                for (int u = 0; u < NS; ++u)
+                {
+                    const float pv = expf(sv[u] - mn);                         // masked: exp(-inf) = 0
+                    sum += pv;
+                    pw[(g * 4 + i) * PS + u * 16 + c] = from_f<bf16_t>(pv).u;
+                }
                 #pragma unroll
                 for (int o = 8; o > 0; o >>= 1) sum += __shfl_xor(sum, o, 64);
                 corr[i] = expf(m[i] - mn);
                 l[i] = l[i] * corr[i] + sum;
                 m[i] = mn;
-                pw[(g * 4 + i) * PS + c] = from_f<bf16_t>(pa).u;
-                pw[(g * 4 + i) * PS + 16 + c] = from_f<bf16_t>(pb).u;
             }
             #pragma unroll
             for (int t = 0; t < NV; ++t)
@@ -142,12 +156,16 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(bf16_t* __restri
                 for (int i = 0; i < 4; ++i) acc[t][i] *= corr[i];
             }
             __builtin_amdgcn_wave_barrier();                                   // LDS serves a wave's accesses in order: its own P stores are visible to the reads below
-            const bf16x8 pa8 = *(const bf16x8*) (pw + c * PS + g * 8);
             #pragma unroll
-            for (int t = 0; t < NV; ++t)
+            for (int kk = 0; kk < AM_KEYS / 32; ++kk)
             {
-                const bf16x8 vb = *(const bf16x8*) (vt_lds + (t * 16 + c) * VS + g * 8);
-                acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pa8, vb, acc[t], 0, 0, 0);
+                const bf16x8 pa8 = *(const bf16x8*) (pw + c * PS + kk * 32 + g * 8);
+                #pragma unroll
+                for (int t = 0; t < NV; ++t)
+                {
+                    const bf16x8 vb = *(const bf16x8*) (vt_lds + (t * 16 + c) * VS + kk * 32 + g * 8);
+                    acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pa8, vb, acc[t], 0, 0, 0);
+                }
             }
         }
     }
@@ -182,14 +200,16 @@ extern "C" int exl3_mix_attn_prefill_mfma(void* out, const void* q, int64_t q_ld
     const dim3 grid((max_rows + AM_ROWS - 1) / AM_ROWS, batch, heads);
     const int k_vec = ((uintptr_t) k % 16 == 0) && (k_ld % 8 == 0) && (dim % 8 == 0);
     const int v_vec = ((uintptr_t) v_norm % 16 == 0) && (vdim % 8 == 0);
-    #define AM_LAUNCH(KDV, NVV) do { \
-        const size_t sm = (size_t) (AM_KEYS * (KDV * 32 + AM_PAD) + NVV * 16 * (AM_KEYS + AM_PAD) + 4 * 16 * (AM_KEYS + AM_PAD)) * sizeof(uint16_t); \
-        hipLaunchKernelGGL((attn_prefill_mfma_kernel<KDV, NVV>), grid, dim3(256), sm, (hipStream_t) stream, (bf16_t*) out, (const bf16_t*) q, q_ld, (const bf16_t*) k, k_ld, \
-                           (const bf16_t*) v_norm, (const bf16_t*) gate, gate_ld, sink, cu, heads, kv_heads, dim, vdim, scale, window, k_vec, v_vec); } while (0)
+    #define AM_LDS(KDV, NVV, KTV) ((size_t) (KTV * (KDV * 32 + AM_PAD) + NVV * 16 * (KTV + AM_PAD) + (AM_THREADS / 64) * 16 * (KTV + AM_PAD)) * sizeof(uint16_t))
+    #define AM_LAUNCH(KDV, NVV, KTV) do { \
+        static_assert(AM_LDS(KDV, NVV, KTV) <= 65536, "tile does not fit the LDS"); \
+        hipLaunchKernelGGL((attn_prefill_mfma_kernel<KDV, NVV, KTV>), grid, dim3(AM_THREADS), AM_LDS(KDV, NVV, KTV), (hipStream_t) stream, (bf16_t*) out, (const bf16_t*) q, q_ld, \
+                           (const bf16_t*) k, k_ld, (const bf16_t*) v_norm, (const bf16_t*) gate, gate_ld, sink, cu, heads, kv_heads, dim, vdim, scale, window, k_vec, v_vec); } while (0)
     const int kd = (dim + 31) / 32, nv = (vdim + 15) / 16;
-    if (kd <= 2)      { if (nv <= 4) AM_LAUNCH(2, 4); else if (nv <= 8) AM_LAUNCH(2, 8); else AM_LAUNCH(2, 16); }
-    else if (kd <= 4) { if (nv <= 4) AM_LAUNCH(4, 4); else if (nv <= 8) AM_LAUNCH(4, 8); else AM_LAUNCH(4, 16); }
-    else              { if (nv <= 4) AM_LAUNCH(8, 4); else if (nv <= 8) AM_LAUNCH(8, 8); else AM_LAUNCH(8, 16); }
+    if (kd <= 2)      { if (nv <= 4) AM_LAUNCH(2, 4, 64); else if (nv <= 8) AM_LAUNCH(2, 8, 64); else AM_LAUNCH(2, 16, 64); }
+    else if (kd <= 4) { if (nv <= 4) AM_LAUNCH(4, 4, 64); else if (nv <= 8) AM_LAUNCH(4, 8, 64); else AM_LAUNCH(4, 16, 32); }
+    else              { if (nv <= 4) AM_LAUNCH(8, 4, 64); else if (nv <= 8) AM_LAUNCH(8, 8, 32); else AM_LAUNCH(8, 16, 32); }
+    #undef AM_LDS
     #undef AM_LAUNCH
     return mix_check_launch("mix_attn_prefill_mfma");
 }
