@@ -98,7 +98,18 @@ __device__ __forceinline__ void attn_row(T* __restrict__ out, const T* __restric
             const int c = lane + 64 * i;
             float a = acc[i] * corr;
             if (c < vdim)
-                for (int jj = 0; jj < cnt; ++jj) a += pw[jj] * to_f(vb[(int64_t) (j0 + jj) * v_step + c]);
+            {
+                int jj = 0;
+                for (; jj + 8 <= cnt; jj += 8)                // eight value rows in flight, then the sums
+                {
+                    float vv[8];
+                    #pragma unroll
+                    for (int e = 0; e < 8; ++e) vv[e] = to_f(vb[(int64_t) (j0 + jj + e) * v_step + c]);
+                    #pragma unroll
+                    for (int e = 0; e < 8; ++e) a += pw[jj + e] * vv[e];
+                }
+                for (; jj < cnt; ++jj) a += pw[jj] * to_f(vb[(int64_t) (j0 + jj) * v_step + c]);
+            }
             acc[i] = a;
         }
         __builtin_amdgcn_wave_barrier();

@@ -72,7 +72,16 @@ __global__ __launch_bounds__(256) void gla_scan_kernel(float* __restrict__ o, fl
             float z = a2_bias ? a2_bias[hc] : 0.f;
             const T* lrow = lr + n * lr_ld;
             const T* arow = a2 + (int64_t) hc * rank;
-            for (int r = 0; r < rank; ++r) z += to_f(lrow[r]) * to_f(arow[r]);
+            int r = 0;
+            for (; r + 8 <= rank; r += 8)                   // eight loads in flight, then the sums (a rolled loop waits for every load in turn)
+            {
+                float a[8], bb[8];
+                #pragma unroll
+                for (int e = 0; e < 8; ++e) { a[e] = to_f(lrow[r + e]); bb[e] = to_f(arow[r + e]); }
+                #pragma unroll
+                for (int e = 0; e < 8; ++e) z += a[e] * bb[e];
+            }
+            for (; r < rank; ++r) z += to_f(lrow[r]) * to_f(arow[r]);
             as[idx] = expf(log_sigmoid_f(z) * inv_tau);
         }
         for (int idx = threadIdx.x; idx < tc * 64; idx += 256)

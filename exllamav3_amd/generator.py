@@ -7,6 +7,12 @@ batch cap become ONE packed prompt step (unequal prompt lengths, no padding), an
 advances by one token in one decode step, whatever step they were admitted in.  A job that ends (token budget, stop token) gives its
 slot back at once and the next admission reuses it.
 
+Decode steps as graphs.  On a GPU the decode step of a given batch size is captured into a hipGraph the second time that size occurs
+(the first time runs eagerly, which is also the libraries' warm-up) and replayed from then on: the step's integers (tokens, slots,
+positions) are copied into the captured step's own device buffer, everything else -- weights, cache buffers, scratch from the graph's
+pool -- keeps its address.  A cache that grows moves its buffers, and the graphs are dropped.  Prompt steps run eagerly (their shapes
+vary, and the experts of long prompts read their counts on the host).
+
 Sampling.  Greedy when temperature is 0; otherwise temperature, top-k and top-p filtering on the float32 logits and one multinomial
 draw per job from the job's own generator (so a job's tokens do not depend on what else is in the batch).
 """
@@ -63,12 +69,46 @@ class Job:
 
 
 class Generator:
-    def __init__(self, model, cache: SlotStateCache | None = None, max_batch: int = 64, max_step_rows: int = 16384):
+    def __init__(self, model, cache: SlotStateCache | None = None, max_batch: int = 64, max_step_rows: int = 16384, graphs: bool | None = None):
         self.model = model
         self.cache = cache if cache is not None else model.new_cache()
         self.max_batch, self.max_step_rows = max_batch, max_step_rows
         self.waiting: list[Job] = []
         self.running: list[Job] = []
+        self.graphs = (torch.device(model.device).type == "cuda") if graphs is None else graphs
+        self._graphs: dict[int, tuple] = {}      # batch size -> (graph, its StepBatch, its logits)
+        self._seen: set[int] = set()
+        self._generation = self.cache.generation
+        self.graph_replays = 0
+
+    def _decode_step(self, entries) -> torch.Tensor:
+        """One token per sequence: eager the first time a batch size occurs, captured the second time, replayed afterwards."""
+        if not self.graphs:
+            return self.model.step(self.cache.begin_step(entries), self.cache)
+        if self._generation != self.cache.generation:
+            self._graphs.clear(); self._seen.clear()
+            self._generation = self.cache.generation
+        b = len(entries)
+        held = self._graphs.get(b)
+        if held is not None:
+            graph, sb, logits = held
+            self.cache.begin_step(entries, into=sb)
+            graph.replay()
+            self.graph_replays += 1
+            return logits
+        sb = self.cache.begin_step(entries)
+        if not sb.decode or b not in self._seen:
+            self._seen.add(b)
+            return self.model.step(sb, self.cache)
+        # capture records the launches without running them; the replay right after is this step
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            logits = self.model.step(sb, self.cache)
+        self._graphs[b] = (graph, sb, logits)
+        graph.replay()
+        self.graph_replays += 1
+        return logits
 
     def enqueue(self, job: Job) -> Job:
         if not job.prompt:
@@ -102,8 +142,10 @@ class Generator:
             jobs, entries = list(self.running), [(j.slot, [j.output[-1]]) for j in self.running]
         else:
             return []
-        sb = self.cache.begin_step(entries)
-        logits = self.model.step(sb, self.cache)
+        if new:
+            logits = self.model.step(self.cache.begin_step(entries), self.cache)
+        else:
+            logits = self._decode_step(entries)
         out = []
         for i, j in enumerate(jobs):
             t = j._sampler.sample(logits[i])

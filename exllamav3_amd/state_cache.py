@@ -36,6 +36,7 @@ class StepBatch:
     len_after: torch.Tensor     # int32 [batch], length after the step
     want_rows: torch.Tensor | None = None     # int32 [m]: rows whose logits are asked for (may be empty)
     host_lens: list = field(default_factory=list)
+    buffer: torch.Tensor | None = None        # the one device array that the tensors above are views of
 
 
 class SlotStateCache:
@@ -46,6 +47,7 @@ class SlotStateCache:
         self.layers: list[dict[str, torch.Tensor]] = [dict() for _ in layer_specs]
         self.free: list[int] = []
         self.length: dict[int, int] = {}         # slot -> tokens held by the sequence that owns it
+        self.generation = 0
         self._grow(max(1, slots))
 
     def bytes_per_slot(self) -> int:
@@ -68,6 +70,7 @@ class SlotStateCache:
                 self.layers[li][s.name] = buf
         self.free.extend(range(new_capacity - 1, self.capacity - 1, -1))      # lowest number on top of the stack
         self.capacity = new_capacity
+        self.generation += 1                   # the buffers moved: whoever holds their addresses (captured graphs) starts over
 
     def alloc(self) -> int:
         if not self.free:
@@ -85,9 +88,11 @@ class SlotStateCache:
     def in_use(self) -> int:
         return len(self.length)
 
-    def begin_step(self, entries: list[tuple[int, list[int]]], want: list[list[int]] | None = None) -> StepBatch:
+    def begin_step(self, entries: list[tuple[int, list[int]]], want: list[list[int]] | None = None, into: StepBatch | None = None) -> StepBatch:
         """entries: (slot, the sequence's next tokens).  Either every sequence is at position 0 (a prompt step) or every sequence brings one
-        token (a decode step).  want: per entry, the places among its tokens whose logits are asked for (None: every sequence's last)."""
+        token (a decode step).  want: per entry, the places among its tokens whose logits are asked for (None: every sequence's last).
+        into: a StepBatch of the same layout (same row and sequence counts) whose device buffer is overwritten in place -- a captured graph keeps
+        reading the same addresses."""
         lens = [len(t) for _, t in entries]
         if not entries or min(lens) < 1:
             raise RuntimeError("a step needs at least one token per sequence")
@@ -112,11 +117,20 @@ class SlotStateCache:
             rows = [cu[i] + p for i, w in enumerate(want) for p in w]
         # one host array, one copy: the pieces are views of it on the device
         flat = tokens + cu + tok_seq + tok_pos + slots + pos0 + after + rows
-        dev = torch.tensor(flat, dtype=torch.int32).to(self.device, non_blocking=False)
+        host = torch.tensor(flat, dtype=torch.int32)
+        if into is not None:
+            if (into.n, into.batch, into.decode, into.want_rows.numel()) != (n, b, decode, len(rows)) or into.buffer.numel() != len(flat):
+                raise RuntimeError("begin_step(into=...): the step has another layout than the one the buffer was made for")
+            into.buffer.copy_(host)
+            for (s, _), a in zip(entries, after):
+                self.length[s] = a
+            into.host_lens = lens
+            return into
+        dev = host.to(self.device, non_blocking=False)
         cuts, at = [], 0
         for ln in (n, b + 1, n, n, b, b, b, len(rows)):
             cuts.append(dev[at: at + ln]); at += ln
         for (s, _), a in zip(entries, after):
             self.length[s] = a
         return StepBatch(n=n, batch=b, decode=decode, max_rows=max(lens), tokens=cuts[0], cu=cuts[1], tok_seq=cuts[2], tok_pos=cuts[3], slots=cuts[4],
-                         pos0=cuts[5], len_after=cuts[6], want_rows=cuts[7], host_lens=lens)
+                         pos0=cuts[5], len_after=cuts[6], want_rows=cuts[7], host_lens=lens, buffer=dev)

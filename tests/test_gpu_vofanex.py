@@ -369,3 +369,31 @@ def test_greedy_generation_through_the_scheduler_matches_oracle(models, name):
     got = gen.generate(prompts, max_new_tokens=new)
     assert got == want
     assert gen.cache.in_use() == 0
+
+
+def test_decode_graphs_replay_bit_for_bit_what_eager_steps_compute(models):
+    """The generator captures the decode step of a batch size the second time it occurs and replays it afterwards.  Two generators over the same
+    jobs, one eager and one with graphs, are stepped side by side (so eager work and synchronisations lie between the replays): every step's
+    sampled tokens are equal, and the logits of every replayed step equal the eager step's bit for bit.  Jobs end at different times, so several batch
+    sizes are captured, and the moe layers' decode path (no host read) is inside the graph."""
+    from exllamav3_amd.generator import Generator, Job
+    orc, ms, vocab = models["c"]
+    for dt in (torch.float32, torch.bfloat16):
+        m = ms[dt]
+        prompts = [toks(vocab, n, 70 + n) for n in (9, 4, 15)]
+        lens = [30, 12, 21]
+        ge, gg = Generator(m, cache=m.new_cache(4), graphs=False), Generator(m, cache=m.new_cache(4), graphs=True)
+        seen = {"e": [], "g": []}
+        for gen, key in ((ge, "e"), (gg, "g")):
+            inner = gen._decode_step
+            gen._decode_step = (lambda entries, inner=inner, key=key: seen[key].append(inner(entries).clone()) or seen[key][-1])
+            for p, n in zip(prompts, lens):
+                gen.enqueue(Job(list(p), n))
+        while ge.busy() or gg.busy():
+            a, b = ge.iterate(), gg.iterate()
+            torch.cuda.synchronize()
+            assert [t for _, t in a] == [t for _, t in b]
+        assert gg.graph_replays >= 20 and len(gg._graphs) == 3 and ge.graph_replays == 0
+        assert len(seen["e"]) == len(seen["g"])
+        for x, y in zip(seen["e"], seen["g"]):
+            assert torch.equal(x, y)
