@@ -3,14 +3,20 @@
 // more term of the denominator and nothing else.
 //
 // One workgroup = 128 query rows of one sequence and one head, 8 waves of 16 rows.  Key tiles of KT = 64 rows (32 for the largest heads, where
-// 64 would not fit 64 KB of LDS) are staged in LDS once for the eight waves: K as stored, V transposed (so that both are read as 16-byte contraction groups).  MFMA operand lane (g = lane / 16, c = lane % 16)
-// holds row / column c and contraction slots 8g .. 8g+7; result lane (g, c) holds rows 4g .. 4g+3 of column c.  A wave's P tile goes
-// through its own LDS patch from the result layout to the operand layout.  Only the key tiles that intersect the window of the block's
-// rows are visited, and a wave skips the tiles outside its own rows' windows.
+// 64 would not fit 64 KB of LDS) are staged in LDS once for the eight waves: K as stored, V transposed (value column, key).
+//
+// MFMA operand lane (g = lane / 16, c = lane % 16) holds row / column c and contraction slots 8g .. 8g+7; result lane (g, c) holds rows
+// 4g .. 4g+3 of column c.  The scores are computed TRANSPOSED, S^T = K Q^T (keys are rows, the wave's 16 queries are columns): a lane then
+// holds scores of ONE query (column c), so the running maximum, the sum and the rescale factor are per-lane scalars (two cross-lane steps
+// per tile for the maximum, the sum is reduced once at the end), and the result registers of two 16-key tiles are, as they stand, the B
+// operand of O^T = V^T P^T when contraction slot (g, e) is read as key 4g + e of the first tile (e < 4) or of the second (e >= 4); the A operand
+// V^T is read from LDS in the same key order (two 8-byte reads).  No probability goes through LDS.  Only the key tiles that intersect the
+// window of the block's rows are visited, and a wave skips the tiles outside its own rows' windows.
 #include "mix_common.cuh"
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 
 #define AM_ROWS 128
 #define AM_THREADS 512
@@ -23,11 +29,10 @@ __global__ __launch_bounds__(AM_THREADS) void attn_prefill_mfma_kernel(bf16_t* _
                                                                 const float* __restrict__ sink, const int32_t* __restrict__ cu,
                                                                 int heads, int kv_heads, int dim, int vdim, float scale, int window, int k_vec, int v_vec)
 {
-    constexpr int DP = KD * 32, KS = DP + AM_PAD, VS = AM_KEYS + AM_PAD, PS = AM_KEYS + AM_PAD;
+    constexpr int DP = KD * 32, KS = DP + AM_PAD, VS = AM_KEYS + AM_PAD;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     uint16_t* k_lds = (uint16_t*) smem_raw;                       // [AM_KEYS][KS]
     uint16_t* vt_lds = k_lds + AM_KEYS * KS;                      // [NV * 16][VS]   (value column, key)
-    uint16_t* p_lds = vt_lds + NV * 16 * VS;                      // [8 waves][16][PS]
 
     const int b = blockIdx.y, h = blockIdx.z;
     const int first = cu[b], len = cu[b + 1] - first;
@@ -35,9 +40,8 @@ __global__ __launch_bounds__(AM_THREADS) void attn_prefill_mfma_kernel(bf16_t* _
     if (q0 >= len) return;
     const int kvh = h / (heads / kv_heads);
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6, g = lane >> 4, c = lane & 15;
-    uint16_t* pw = p_lds + w * 16 * PS;
 
-    // this wave's 16 query rows as A operands (rows beyond the sequence read row len-1: computed and never stored)
+    // this wave's 16 query rows as B operands of S^T = K Q^T (rows beyond the sequence read row len-1: computed and never stored)
     const int qrow_a = min(q0 + w * 16 + c, len - 1);
     bf16x8 qf[KD];
     #pragma unroll
@@ -55,11 +59,11 @@ __global__ __launch_bounds__(AM_THREADS) void attn_prefill_mfma_kernel(bf16_t* _
     const int wq_lo = q0 + w * 16, wq_hi = min(q0 + w * 16 + 15, len - 1);           // this wave's rows
     const bool wave_live = wq_lo < len;
 
-    const float sk = sink ? sink[h] : -1e30f;
-    float m[4], l[4];
-    f32x4 acc[NV];
-    #pragma unroll
-    for (int i = 0; i < 4; ++i) { m[i] = sk; l[i] = sink ? 1.0f : 0.0f; }
+    // per lane: query c of the wave.  m: running maximum (the same in the four lanes of a query), l: this lane's share of the sum
+    const int qi = q0 + w * 16 + c;
+    float m = sink ? sink[h] : -1e30f;
+    float l = (sink && g == 0) ? 1.0f : 0.0f;
+    f32x4 acc[NV];                                                 // O^T tiles: value rows 4g .. 4g+3 of tile t, query c
     #pragma unroll
     for (int t = 0; t < NV; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
 
@@ -114,74 +118,73 @@ __global__ __launch_bounds__(AM_THREADS) void attn_prefill_mfma_kernel(bf16_t* _
                 for (int u = 0; u < NS; ++u)
                 {
                     const bf16x8 kf = *(const bf16x8*) (k_lds + (u * 16 + c) * KS + s * 32 + g * 8);
-                    sc[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[s], kf, sc[u], 0, 0, 0);
+                    sc[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[s], sc[u], 0, 0, 0);
                 }
             }
-            float corr[4];
+            // sc[u][i] = score of key j0 + 16u + 4g + i against query qi
+            float mx = -INFINITY;
             #pragma unroll
-            for (int i = 0; i < 4; ++i)
+            for (int u = 0; u < NS; ++u)
             {
-                const int qi = q0 + w * 16 + g * 4 + i;                       // this result row's position
-                float sv[NS];
-                float mx = -INFINITY;
                 #pragma unroll
-                for (int u = 0; u < NS; ++u)
+                for (int i = 0; i < 4; ++i)
                 {
-                    const int j = j0 + u * 16 + c;
+                    const int j = j0 + u * 16 + g * 4 + i;
                     const bool ok = j <= qi && qi - j < window && qi < len;
-                    sv[u] = ok ? sc[u][i] * scale : -INFINITY;
-                    mx = fmaxf(mx, sv[u]);
+                    sc[u][i] = ok ? sc[u][i] * scale : -INFINITY;
+                    mx = fmaxf(mx, sc[u][i]);
                 }
+            }
+            mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+            const float mn = fmaxf(m, mx);                                     // finite: m starts at the sink or at -1e30
+            const float corr = __expf(m - mn);
+            m = mn;
+            float sum = 0.f;
+            #pragma unroll
+            for (int u = 0; u < NS; ++u)
+            {
                 #pragma unroll
-                for (int o = 8; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
-                const float mn = fmaxf(m[i], mx);                              // finite: m starts at the sink or at -1e30
-                float sum = 0.f;
+                for (int i = 0; i < 4; ++i) { sc[u][i] = __expf(sc[u][i] - mn); sum += sc[u][i]; }      // masked: exp(-inf) = 0
+            }
+            l = l * corr + sum;
+            #pragma unroll
+            for (int t = 0; t < NV; ++t) acc[t] *= corr;
+            #pragma unroll
+            for (int kk = 0; kk < NS / 2; ++kk)
+            {
+                union { bf16x8 v; uint16_t u[8]; } pb;
                 #pragma unroll
-                for (int u = 0; u < NS; ++u)
+                for (int i = 0; i < 4; ++i)
                 {
-                    const float pv = expf(sv[u] - mn);                         // masked: exp(-inf) = 0
-                    sum += pv;
-                    pw[(g * 4 + i) * PS + u * 16 + c] = from_f<bf16_t>(pv).u;
+                    pb.u[i] = from_f<bf16_t>(sc[2 * kk][i]).u;
+                    pb.u[4 + i] = from_f<bf16_t>(sc[2 * kk + 1][i]).u;
                 }
-                #pragma unroll
-                for (int o = 8; o > 0; o >>= 1) sum += __shfl_xor(sum, o, 64);
-                corr[i] = expf(m[i] - mn);
-                l[i] = l[i] * corr[i] + sum;
-                m[i] = mn;
-            }
-            #pragma unroll
-            for (int t = 0; t < NV; ++t)
-            {
-                #pragma unroll
-                for (int i = 0; i < 4; ++i) acc[t][i] *= corr[i];
-            }
-            __builtin_amdgcn_wave_barrier();                                   // LDS serves a wave's accesses in order: its own P stores are visible to the reads below
-            #pragma unroll
-            for (int kk = 0; kk < AM_KEYS / 32; ++kk)
-            {
-                const bf16x8 pa8 = *(const bf16x8*) (pw + c * PS + kk * 32 + g * 8);
                 #pragma unroll
                 for (int t = 0; t < NV; ++t)
                 {
-                    const bf16x8 vb = *(const bf16x8*) (vt_lds + (t * 16 + c) * VS + kk * 32 + g * 8);
-                    acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pa8, vb, acc[t], 0, 0, 0);
+                    union { bf16x8 v; bf16x4 h[2]; } va;
+                    va.h[0] = *(const bf16x4*) (vt_lds + (t * 16 + c) * VS + (2 * kk) * 16 + g * 4);
+                    va.h[1] = *(const bf16x4*) (vt_lds + (t * 16 + c) * VS + (2 * kk + 1) * 16 + g * 4);
+                    acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va.v, pb.v, acc[t], 0, 0, 0);
                 }
             }
         }
     }
     if (!wave_live) return;
+    l += __shfl_xor(l, 16, 64);
+    l += __shfl_xor(l, 32, 64);
+    if (qi >= len) return;
+    const int64_t n = first + qi;
+    const float gt = gate ? sigmoid_f(to_f(gate[n * gate_ld + h])) : 1.0f;
+    const float f = (l > 0.f ? 1.0f / l : 0.f) * gt;
     #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int t = 0; t < NV; ++t)
     {
-        const int qi = q0 + w * 16 + g * 4 + i;
-        if (qi >= len) continue;
-        const int64_t n = first + qi;
-        const float gt = gate ? sigmoid_f(to_f(gate[n * gate_ld + h])) : 1.0f;
-        const float f = (l[i] > 0.f ? 1.0f / l[i] : 0.f) * gt;
         #pragma unroll
-        for (int t = 0; t < NV; ++t)
+        for (int i = 0; i < 4; ++i)
         {
-            const int col = t * 16 + c;
+            const int col = t * 16 + g * 4 + i;
             if (col < vdim) out[(n * heads + h) * vdim + col] = from_f<bf16_t>(acc[t][i] * f);
         }
     }
@@ -200,15 +203,15 @@ extern "C" int exl3_mix_attn_prefill_mfma(void* out, const void* q, int64_t q_ld
     const dim3 grid((max_rows + AM_ROWS - 1) / AM_ROWS, batch, heads);
     const int k_vec = ((uintptr_t) k % 16 == 0) && (k_ld % 8 == 0) && (dim % 8 == 0);
     const int v_vec = ((uintptr_t) v_norm % 16 == 0) && (vdim % 8 == 0);
-    #define AM_LDS(KDV, NVV, KTV) ((size_t) (KTV * (KDV * 32 + AM_PAD) + NVV * 16 * (KTV + AM_PAD) + (AM_THREADS / 64) * 16 * (KTV + AM_PAD)) * sizeof(uint16_t))
+    #define AM_LDS(KDV, NVV, KTV) ((size_t) (KTV * (KDV * 32 + AM_PAD) + NVV * 16 * (KTV + AM_PAD)) * sizeof(uint16_t))
     #define AM_LAUNCH(KDV, NVV, KTV) do { \
         static_assert(AM_LDS(KDV, NVV, KTV) <= 65536, "tile does not fit the LDS"); \
         hipLaunchKernelGGL((attn_prefill_mfma_kernel<KDV, NVV, KTV>), grid, dim3(AM_THREADS), AM_LDS(KDV, NVV, KTV), (hipStream_t) stream, (bf16_t*) out, (const bf16_t*) q, q_ld, \
                            (const bf16_t*) k, k_ld, (const bf16_t*) v_norm, (const bf16_t*) gate, gate_ld, sink, cu, heads, kv_heads, dim, vdim, scale, window, k_vec, v_vec); } while (0)
     const int kd = (dim + 31) / 32, nv = (vdim + 15) / 16;
     if (kd <= 2)      { if (nv <= 4) AM_LAUNCH(2, 4, 64); else if (nv <= 8) AM_LAUNCH(2, 8, 64); else AM_LAUNCH(2, 16, 64); }
-    else if (kd <= 4) { if (nv <= 4) AM_LAUNCH(4, 4, 64); else if (nv <= 8) AM_LAUNCH(4, 8, 64); else AM_LAUNCH(4, 16, 32); }
-    else              { if (nv <= 4) AM_LAUNCH(8, 4, 64); else if (nv <= 8) AM_LAUNCH(8, 8, 32); else AM_LAUNCH(8, 16, 32); }
+    else if (kd <= 4) { if (nv <= 4) AM_LAUNCH(4, 4, 64); else if (nv <= 8) AM_LAUNCH(4, 8, 64); else AM_LAUNCH(4, 16, 64); }
+    else              { if (nv <= 4) AM_LAUNCH(8, 4, 64); else if (nv <= 8) AM_LAUNCH(8, 8, 64); else AM_LAUNCH(8, 16, 32); }
     #undef AM_LDS
     #undef AM_LAUNCH
     return mix_check_launch("mix_attn_prefill_mfma");
