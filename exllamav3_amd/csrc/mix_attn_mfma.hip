@@ -21,6 +21,7 @@ typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 #define AM_ROWS 128
 #define AM_THREADS 512
 #define AM_PAD 8
+#define LOG2E 1.4426950408889634f
 
 // KD: contraction steps of 32 over the (zero-padded) head dim; NV: 16-column tiles of the (padded) value dim.
 template <int KD, int NV, int AM_KEYS>
@@ -121,31 +122,47 @@ __global__ __launch_bounds__(AM_THREADS) void attn_prefill_mfma_kernel(bf16_t* _
                     sc[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[s], sc[u], 0, 0, 0);
                 }
             }
-            // sc[u][i] = score of key j0 + 16u + 4g + i against query qi
+            // sc[u][i] = raw score of key j0 + 16u + 4g + i against query qi.  A tile whose keys all lie inside the window of every row of the wave
+            // needs no mask (wave-uniform branch; with a window of many tiles that is most of them).
+            const bool interior = j0 + AM_KEYS - 1 <= wq_lo && wq_hi - j0 < window && q0 + w * 16 + 15 < len;
             float mx = -INFINITY;
-            #pragma unroll
-            for (int u = 0; u < NS; ++u)
+            if (interior)
             {
                 #pragma unroll
-                for (int i = 0; i < 4; ++i)
+                for (int u = 0; u < NS; ++u)
                 {
-                    const int j = j0 + u * 16 + g * 4 + i;
-                    const bool ok = j <= qi && qi - j < window && qi < len;
-                    sc[u][i] = ok ? sc[u][i] * scale : -INFINITY;
-                    mx = fmaxf(mx, sc[u][i]);
+                    #pragma unroll
+                    for (int i = 0; i < 4; ++i) mx = fmaxf(mx, sc[u][i]);
+                }
+            }
+            else
+            {
+                #pragma unroll
+                for (int u = 0; u < NS; ++u)
+                {
+                    #pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                    {
+                        const int j = j0 + u * 16 + g * 4 + i;
+                        const bool ok = j <= qi && qi - j < window && qi < len;
+                        sc[u][i] = ok ? sc[u][i] : -INFINITY;
+                        mx = fmaxf(mx, sc[u][i]);
+                    }
                 }
             }
             mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
             mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-            const float mn = fmaxf(m, mx);                                     // finite: m starts at the sink or at -1e30
-            const float corr = __expf(m - mn);
+            const float mn = fmaxf(m, mx * scale);                             // scale > 0 (host-checked): the largest raw score is the largest score
+            const float corr = __builtin_amdgcn_exp2f((m - mn) * LOG2E);
             m = mn;
+            // weight = exp(score * scale - m) = 2^(score * c2 - m * log2 e): one multiply-add and one v_exp_f32 per key
+            const float c2 = scale * LOG2E, off = -mn * LOG2E;
             float sum = 0.f;
             #pragma unroll
             for (int u = 0; u < NS; ++u)
             {
                 #pragma unroll
-                for (int i = 0; i < 4; ++i) { sc[u][i] = __expf(sc[u][i] - mn); sum += sc[u][i]; }      // masked: exp(-inf) = 0
+                for (int i = 0; i < 4; ++i) { sc[u][i] = __builtin_amdgcn_exp2f(sc[u][i] * c2 + off); sum += sc[u][i]; }      // masked: 2^(-inf) = 0
             }
             l = l * corr + sum;
             #pragma unroll
@@ -153,12 +170,12 @@ __global__ __launch_bounds__(AM_THREADS) void attn_prefill_mfma_kernel(bf16_t* _
             #pragma unroll
             for (int kk = 0; kk < NS / 2; ++kk)
             {
-                union { bf16x8 v; uint16_t u[8]; } pb;
+                bf16x8 pb;
                 #pragma unroll
                 for (int i = 0; i < 4; ++i)
                 {
-                    pb.u[i] = from_f<bf16_t>(sc[2 * kk][i]).u;
-                    pb.u[4 + i] = from_f<bf16_t>(sc[2 * kk + 1][i]).u;
+                    pb[i] = (__bf16) sc[2 * kk][i];
+                    pb[4 + i] = (__bf16) sc[2 * kk + 1][i];
                 }
                 #pragma unroll
                 for (int t = 0; t < NV; ++t)
@@ -166,7 +183,7 @@ __global__ __launch_bounds__(AM_THREADS) void attn_prefill_mfma_kernel(bf16_t* _
                     union { bf16x8 v; bf16x4 h[2]; } va;
                     va.h[0] = *(const bf16x4*) (vt_lds + (t * 16 + c) * VS + (2 * kk) * 16 + g * 4);
                     va.h[1] = *(const bf16x4*) (vt_lds + (t * 16 + c) * VS + (2 * kk + 1) * 16 + g * 4);
-                    acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va.v, pb.v, acc[t], 0, 0, 0);
+                    acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va.v, pb, acc[t], 0, 0, 0);
                 }
             }
         }
@@ -198,6 +215,7 @@ extern "C" int exl3_mix_attn_prefill_mfma(void* out, const void* q, int64_t q_ld
     MIX_CHECK(batch >= 0 && max_rows >= 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && heads <= 65535 && batch <= 65535,
               "mix_attn_prefill_mfma: heads %d / kv_heads %d / batch %d", heads, kv_heads, batch);
     MIX_CHECK(dim > 0 && dim <= 256 && vdim > 0 && vdim <= 256 && window > 0, "mix_attn_prefill_mfma: dim %d and vdim %d must be <= 256", dim, vdim);
+    MIX_CHECK(scale > 0.f, "mix_attn_prefill_mfma: the score scale must be positive (the running maximum is taken over raw scores)");
     MIX_CHECK(q_ld >= (int64_t) heads * dim && k_ld >= (int64_t) kv_heads * dim && (!gate || gate_ld >= heads), "mix_attn_prefill_mfma: bad row strides");
     if (batch == 0 || max_rows == 0) return EXL3_MIX_OK;
     const dim3 grid((max_rows + AM_ROWS - 1) / AM_ROWS, batch, heads);

@@ -14,11 +14,9 @@ __device__ __forceinline__ float to_f(float v) { return v; }
 template <typename T> __device__ __forceinline__ T from_f(float f);
 template <> __device__ __forceinline__ bf16_t from_f<bf16_t>(float f)
 {
-    uint32_t u = __float_as_uint(f);
+    const __bf16 h = (__bf16) f;                     // the hardware's conversion: round to nearest, ties to even
     bf16_t r;
-    if ((u & 0x7fffffffu) > 0x7f800000u) { r.u = 0x7fc0; return r; }
-    u += 0x7fffu + ((u >> 16) & 1u);                 // round to nearest, ties to even
-    r.u = (uint16_t) (u >> 16);
+    __builtin_memcpy(&r.u, &h, sizeof(r.u));
     return r;
 }
 template <> __device__ __forceinline__ float from_f<float>(float f) { return f; }

@@ -113,7 +113,7 @@ def attn_prefill(out, q_view, k_view, v_norm, gate_view, sink, cu, tok_seq, tok_
     if sink is not None:
         _f32c(sink, "sink"); _req(sink.numel() == heads, "attn_prefill: sink")
     if mfma is None:
-        mfma = out.dtype == torch.bfloat16 and max_rows >= ATTN_MFMA_MIN_ROWS and dim <= 256 and vdim <= 256
+        mfma = out.dtype == torch.bfloat16 and max_rows >= ATTN_MFMA_MIN_ROWS and dim <= 256 and vdim <= 256 and scale > 0
     if mfma:
         _req(out.dtype == torch.bfloat16 and max_rows > 0 and v_norm.is_contiguous(), "attn_prefill: the matrix-core kernel takes bfloat16 and the step's longest sequence")
         _check(_lib.mixlib().exl3_mix_attn_prefill_mfma(_p(out), _p(q_view), _view(q_view, heads * dim, "q"), _p(k_view), _view(k_view, kv_heads * dim, "k"), _p(v_norm),
