@@ -3,9 +3,49 @@
 // activation between them and the weighted un-sort are the two small kernels at the end of this file.
 #include "mix_common.cuh"
 
+template <typename T> struct vecn;
+template <> struct vecn<bf16_t> { static constexpr int N = 8; };
+template <> struct vecn<float> { static constexpr int N = 4; };
+
+// dot products of one activation row with up to two weight rows, 16 bytes per lane and load (rows 16-byte aligned, length a multiple of the vector)
+template <typename T, bool TWO>
+__device__ __forceinline__ void dot_rows(const T* __restrict__ x, const T* __restrict__ a, const T* __restrict__ b, int len, bool vec, float& ra, float& rb)
+{
+    constexpr int VN = vecn<T>::N;
+    const int lane = threadIdx.x & 63;
+    float sa = 0.f, sb = 0.f;
+    if (vec)
+    {
+        for (int c = lane * VN; c < len; c += 64 * VN)
+        {
+            union { uint4 v; T e[VN]; } tx, ta, tb;
+            tx.v = *(const uint4*) (x + c); ta.v = *(const uint4*) (a + c);
+            if (TWO) tb.v = *(const uint4*) (b + c);
+            #pragma unroll
+            for (int e = 0; e < VN; ++e)
+            {
+                const float xv = to_f(tx.e[e]);
+                sa += xv * to_f(ta.e[e]);
+                if (TWO) sb += xv * to_f(tb.e[e]);
+            }
+        }
+    }
+    else
+    {
+        for (int c = lane; c < len; c += 64)
+        {
+            const float xv = to_f(x[c]);
+            sa += xv * to_f(a[c]);
+            if (TWO) sb += xv * to_f(b[c]);
+        }
+    }
+    ra = wave_sum(sa);
+    if (TWO) rb = wave_sum(sb);
+}
+
 template <typename T>
 __global__ __launch_bounds__(256) void moe_gate_up_kernel(T* __restrict__ hid, const T* __restrict__ h, const T* __restrict__ wg, const T* __restrict__ wu,
-                                                          const int32_t* __restrict__ idx, int experts, int ff, int width, int top)
+                                                          const int32_t* __restrict__ idx, int experts, int ff, int width, int top, int vec)
 {
     const int row = blockIdx.x;                              // n * top + r
     const int j = blockIdx.y * 4 + (threadIdx.x >> 6);
@@ -16,16 +56,15 @@ __global__ __launch_bounds__(256) void moe_gate_up_kernel(T* __restrict__ hid, c
     const T* x = h + (int64_t) (row / top) * width;
     const T* g = wg + ((int64_t) e * ff + j) * width;
     const T* u = wu + ((int64_t) e * ff + j) * width;
-    float ag = 0.f, au = 0.f;
-    for (int c = lane; c < width; c += 64) { const float xv = to_f(x[c]); ag += xv * to_f(g[c]); au += xv * to_f(u[c]); }
-    ag = wave_sum(ag); au = wave_sum(au);
+    float ag, au;
+    dot_rows<T, true>(x, g, u, width, vec != 0, ag, au);
     // the two projections leave the matrix product in the activation type before the activation, like any other linear of the model
     if (lane == 0) hid[(int64_t) row * ff + j] = from_f<T>(silu_f(to_f(from_f<T>(ag))) * to_f(from_f<T>(au)));
 }
 
 template <typename T>
 __global__ __launch_bounds__(256) void moe_down_kernel(T* __restrict__ y, const T* __restrict__ hid, const T* __restrict__ wd, const int32_t* __restrict__ idx,
-                                                       const float* __restrict__ wts, int experts, int ff, int width, int top)
+                                                       const float* __restrict__ wts, int experts, int ff, int width, int top, int vec)
 {
     const int n = blockIdx.x;
     const int col = blockIdx.y * 4 + (threadIdx.x >> 6);
@@ -38,9 +77,9 @@ __global__ __launch_bounds__(256) void moe_down_kernel(T* __restrict__ y, const 
         e = e < 0 ? 0 : (e >= experts ? experts - 1 : e);
         const T* hr = hid + ((int64_t) n * top + r) * ff;
         const T* wr = wd + ((int64_t) e * width + col) * ff;
-        float a = 0.f;
-        for (int c = lane; c < ff; c += 64) a += to_f(hr[c]) * to_f(wr[c]);
-        acc += wts[(int64_t) n * top + r] * wave_sum(a);
+        float a, unused;
+        dot_rows<T, false>(hr, wr, wr, ff, vec != 0, a, unused);
+        acc += wts[(int64_t) n * top + r] * a;
     }
     if (lane == 0) y[(int64_t) n * width + col] = from_f<T>(acc);
 }
@@ -88,8 +127,10 @@ extern "C" int exl3_mix_moe_gate_up(void* hid, const void* h, const void* wg, co
 {
     MIX_CHECK(hid && h && wg && wu && idx && n >= 0 && top > 0 && experts > 0 && ff > 0 && width > 0, "mix_moe_gate_up: bad arguments");
     if (n == 0) return EXL3_MIX_OK;
+    const int vn = dtype == EXL3_MIX_BF16 ? 8 : 4;
+    const int vec = width % vn == 0 && (uintptr_t) h % 16 == 0 && (uintptr_t) wg % 16 == 0 && (uintptr_t) wu % 16 == 0;
     MIX_DISPATCH_T(dtype, hipLaunchKernelGGL(moe_gate_up_kernel<T>, dim3(n * top, (ff + 3) / 4), dim3(256), 0, (hipStream_t) stream, (T*) hid, (const T*) h,
-                                             (const T*) wg, (const T*) wu, idx, experts, ff, width, top));
+                                             (const T*) wg, (const T*) wu, idx, experts, ff, width, top, vec));
     return mix_check_launch("mix_moe_gate_up");
 }
 
@@ -98,7 +139,9 @@ extern "C" int exl3_mix_moe_down(void* y, const void* hid, const void* wd, const
 {
     MIX_CHECK(y && hid && wd && idx && wts && n >= 0 && top > 0 && experts > 0 && ff > 0 && width > 0, "mix_moe_down: bad arguments");
     if (n == 0) return EXL3_MIX_OK;
+    const int vn = dtype == EXL3_MIX_BF16 ? 8 : 4;
+    const int vec = ff % vn == 0 && (uintptr_t) hid % 16 == 0 && (uintptr_t) wd % 16 == 0;
     MIX_DISPATCH_T(dtype, hipLaunchKernelGGL(moe_down_kernel<T>, dim3(n, (width + 3) / 4), dim3(256), 0, (hipStream_t) stream, (T*) y, (const T*) hid, (const T*) wd,
-                                             idx, wts, experts, ff, width, top));
+                                             idx, wts, experts, ff, width, top, vec));
     return mix_check_launch("mix_moe_down");
 }
