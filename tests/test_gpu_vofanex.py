@@ -45,7 +45,7 @@ TOL = {torch.float32: 2e-5, torch.bfloat16: 3e-2}
 # ---- mechanisms alone -------------------------------------------------------------------------------------------------------
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("H,G,d,dv,W,lens", [(4, 2, 16, 24, 5, [17, 1, 9]), (3, 3, 40, 72, 64, [70]), (2, 1, 8, 8, 1, [6, 3]), (6, 2, 32, 130, 7, [20]), (2, 1, 96, 96, 37, [150, 66]), (1, 1, 136, 64, 100, [131])])
+@pytest.mark.parametrize("H,G,d,dv,W,lens", [(4, 2, 16, 24, 5, [17, 1, 9]), (3, 3, 40, 72, 64, [70]), (2, 1, 8, 8, 1, [6, 3]), (6, 2, 32, 130, 7, [20]), (2, 1, 96, 96, 37, [150, 66]), (1, 1, 136, 64, 100, [131]), (3, 1, 20, 12, 9, [40, 33])])
 def test_attention_prefill_then_decode_matches_oracle(gpu, dtype, H, G, d, dv, W, lens):
     from exllamav3_amd import mix_ops
     g = torch.Generator().manual_seed(H * 100 + W)
@@ -334,6 +334,34 @@ def test_decoding_batches_and_slot_reuse_do_not_change_logits(models, name):
         assert cache.in_use() == 1
 
 
+def test_long_prompt_at_odd_sizes_runs_the_segmented_and_matrix_core_paths(gpu, tmp_path):
+    """A 600-token prompt beside a 70-token one through a model whose sizes are multiples of nothing convenient: the recurrent layers run in time segments,
+    the bfloat16 attention on the matrix cores with scalar staging, the experts through the expert-sorted products; then both requests are decoded."""
+    from exllamav3_amd.registry import load_model
+    layers = [dict(type="gla", heads=3, dim=40, vdim=56, tau=5.0, rank=6, mlp=("moe", 36, 5, 2)),
+              dict(type="attention", heads=6, kv_heads=2, dim=20, vdim=28, window=50, mlp=("dense", 150)),
+              dict(type="gla", heads=1, dim=24, vdim=200, tau=30.0, rank=2, mlp=None)]
+    cfg, t = mo.random_model(layers, vocab=300, width=88, seed=77)
+    mo.save_model(str(tmp_path), cfg, t)
+    orc = mo.OracleModel(cfg, t)
+    seqs = [toks(300, 610, 5), toks(300, 80, 6)]
+    cuts = [600, 70]
+    refs = [orc.forward(s) for s in seqs]
+    for dt, bar in ((torch.float32, 3e-5), (torch.bfloat16, 6e-2)):
+        m = load_model(str(tmp_path), gpu, dt); cache = m.new_cache(2)
+        slots = [cache.alloc(), cache.alloc()]
+        want = [list(range(0, c, 7)) + [c - 1] for c in cuts]
+        lg = m.step(cache.begin_step([(sl, s[:c]) for sl, s, c in zip(slots, seqs, cuts)], want), cache)
+        got = [[lg[:len(want[0])]], [lg[len(want[0]):]]]
+        rows = [list(want[0]), list(want[1])]
+        for p in range(10):
+            lg = m.step(cache.begin_step([(sl, [s[c + p]]) for sl, s, c in zip(slots, seqs, cuts)], [[0], [0]]), cache)
+            for i in range(2):
+                got[i].append(lg[i: i + 1]); rows[i].append(cuts[i] + p)
+        for i in range(2):
+            assert logit_err(torch.cat(got[i]), refs[i][rows[i]], QUANT[dt]) < bar, f"request {i} {dt}"
+
+
 def test_long_decoding_stays_on_the_oracle(models):
     orc, ms, vocab = models["a"]
     t = toks(vocab, 140, 4)                                  # 4 prompt tokens, 136 decoded: the 6- and 33-token rings wrap many times
@@ -397,3 +425,47 @@ def test_decode_graphs_replay_bit_for_bit_what_eager_steps_compute(models):
         assert len(seen["e"]) == len(seen["g"])
         for x, y in zip(seen["e"], seen["g"]):
             assert torch.equal(x, y)
+
+
+def test_trace_replay_writes_the_same_logits_however_the_tokens_are_cut(models, tmp_path):
+    """TraceSession (what bin/trace_run runs): a request alone in one step, the same request as a prompt step plus single tokens, and the same
+    request batched with another one; the files hold float32 [wanted, vocab] in the order of the entries and of their wanted places, and slots are
+    given back at "end"."""
+    import io, json
+    import numpy as np
+    from exllamav3_amd.trace import TraceSession
+    orc, ms, vocab = models["c"]
+    m = ms[torch.float32]
+    a, b = toks(vocab, 19, 31), toks(vocab, 8, 32)
+    want_a = [0, 5, 11, 17, 18]
+
+    def run(name, steps):
+        out = tmp_path / name
+        out.mkdir()
+        ts = TraceSession(m, str(out))
+        log = io.StringIO()
+        ts.run([json.dumps(s) for s in steps], out=log)
+        assert log.getvalue().split() == [w for s in steps for w in ("done", str(s["step"]))]
+        assert ts.cache.in_use() == 0
+        return {int(f.name.split(".")[0]): np.fromfile(f, dtype="<f4").reshape(-1, vocab) for f in out.iterdir()}
+
+    whole = run("whole", [{"step": 0, "entries": [{"id": "a", "tokens": a, "want": want_a}], "end": ["a"]}])
+    assert list(whole) == [0] and whole[0].shape == (len(want_a), vocab)
+    ref = orc.forward(a)[want_a].numpy()
+    assert np.abs(whole[0] - ref).max() < 3e-5 * np.abs(ref).max() * 10
+    steps = [{"step": 0, "entries": [{"id": "x", "tokens": a[:12], "want": [0, 5, 11]}], "end": []}]
+    for p in range(12, 19):
+        steps.append({"step": p - 11, "entries": [{"id": "x", "tokens": [a[p]], "want": [0] if p in want_a else []}], "end": ["x"] if p == 18 else []})
+    cut = run("decode", steps)
+    assert sorted(cut) == [0, 6, 7]                          # steps without a wanted place write no file
+    assert np.abs(np.concatenate([cut[0], cut[6], cut[7]]) - whole[0]).max() < 1e-4
+    steps = [{"step": 0, "entries": [{"id": "b", "tokens": b[:3], "want": [2]}, {"id": "a", "tokens": a[:12], "want": [0, 5, 11]}], "end": []}]
+    for p in range(7):
+        e = [{"id": "a", "tokens": [a[12 + p]], "want": [0] if 12 + p in want_a else []}]
+        if 3 + p < len(b):
+            e.insert(0, {"id": "b", "tokens": [b[3 + p]], "want": [0] if 3 + p == 7 else []})
+        steps.append({"step": p + 1, "entries": e, "end": (["b"] if 3 + p == 7 else []) + (["a"] if p == 6 else [])})
+    tog = run("together", steps)
+    assert np.abs(np.concatenate([tog[0][1:], tog[6], tog[7]]) - whole[0]).max() < 1e-4
+    refb = orc.forward(b).numpy()
+    assert np.abs(tog[0][0] - refb[2]).max() < 1e-3 and np.abs(tog[5][0] - refb[7]).max() < 1e-3
