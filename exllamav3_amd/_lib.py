@@ -310,3 +310,4 @@ def _declare_mix(l):
     sig("exl3_mix_silu_mul", vp, vp, vp, i64, i32, vp)
     sig("exl3_mix_moe_combine", vp, vp, vp, vp, i32, i32, i32, i32, vp)
     sig("exl3_mix_attn_prefill_mfma", vp, vp, i64, vp, i64, vp, vp, i64, vp, vp, i32, i32, i32, i32, i32, i32, f32, i32, vp)
+    sig("exl3_mix_moe_expert_major", vp, vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, vp)

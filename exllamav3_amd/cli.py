@@ -30,7 +30,12 @@ def _prepare(model_dir: str):
     if arch == "Vofanex":
         hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
         if os.path.exists(hipcc) or shutil.which("hipcc"):
-            _lib.ensure_mix_built()
+            try:
+                _lib.ensure_mix_built()
+            except Exception as e:               # e.g. a checkout that cannot be written: a library that is already there still serves
+                if not os.path.exists(_lib.MIX_LIB_PATH):
+                    raise
+                print(f"exllamav3_amd: could not rebuild libexl3_mix.so ({type(e).__name__}: {e}); using the one that is there", file=sys.stderr)
         _lib.mixlib()
     else:
         _lib.lib()

@@ -105,6 +105,145 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(T* __restrict__ y, con
     }
 }
 
+// Expert-major form for a handful to a few dozen rows: one workgroup per (expert, four outputs).  The rows that chose the expert are listed in
+// LDS first; a wave then reads each 16-byte piece of ITS weight row(s) once and multiplies it with the same piece of up to EM_ROWS listed
+// rows (their activations come from L1 / L2), so an expert's weights are streamed once however many rows use it.  Needs the 16-byte layout.
+#define EM_ROWS 8
+
+__device__ __forceinline__ int em_list_rows(int* list, const int32_t* __restrict__ idx, int n_rows, int e)
+{
+    // wave 0 compacts the matching (row, choice) indices in order; every thread gets the count
+    __shared__ int cnt_s;
+    const int lane = threadIdx.x & 63;
+    if ((threadIdx.x >> 6) == 0)
+    {
+        int c = 0;
+        for (int base = 0; base < n_rows; base += 64)
+        {
+            const int r = base + lane;
+            const bool hit = r < n_rows && idx[r] == e;
+            const unsigned long long mask = __ballot(hit);
+            if (hit) list[c + __popcll(mask & ((1ull << lane) - 1ull))] = r;
+            c += __popcll(mask);
+        }
+        if (lane == 0) cnt_s = c;
+    }
+    __syncthreads();
+    return cnt_s;
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void moe_gate_up_em_kernel(T* __restrict__ hid, const T* __restrict__ h, const T* __restrict__ wg, const T* __restrict__ wu,
+                                                             const int32_t* __restrict__ idx, int n_rows, int ff, int width, int top)
+{
+    extern __shared__ int em_list[];
+    constexpr int VN = vecn<T>::N;
+    const int e = blockIdx.x, j = blockIdx.y * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+    const int cnt = em_list_rows(em_list, idx, n_rows, e);
+    if (cnt == 0 || j >= ff) return;
+    const T* g = wg + ((int64_t) e * ff + j) * width;
+    const T* u = wu + ((int64_t) e * ff + j) * width;
+    for (int r0 = blockIdx.z * EM_ROWS; r0 < cnt; r0 += gridDim.z * EM_ROWS)      // a long list is shared by the workgroups along z
+    {
+        float sa[EM_ROWS], sb[EM_ROWS];
+        #pragma unroll
+        for (int m = 0; m < EM_ROWS; ++m) { sa[m] = 0.f; sb[m] = 0.f; }
+        for (int c = lane * VN; c < width; c += 64 * VN)
+        {
+            union { uint4 v; T e[VN]; } tg, tu;
+            tg.v = *(const uint4*) (g + c); tu.v = *(const uint4*) (u + c);
+            #pragma unroll
+            for (int m = 0; m < EM_ROWS; ++m)
+            {
+                if (r0 + m < cnt)
+                {
+                    union { uint4 v; T e[VN]; } tx;
+                    tx.v = *(const uint4*) (h + (int64_t) (em_list[r0 + m] / top) * width + c);
+                    #pragma unroll
+                    for (int q = 0; q < VN; ++q)
+                    {
+                        const float xv = to_f(tx.e[q]);
+                        sa[m] += xv * to_f(tg.e[q]); sb[m] += xv * to_f(tu.e[q]);
+                    }
+                }
+            }
+        }
+        #pragma unroll
+        for (int m = 0; m < EM_ROWS; ++m)
+        {
+            if (r0 + m < cnt)
+            {
+                const float ag = wave_sum(sa[m]), au = wave_sum(sb[m]);
+                if (lane == 0) hid[(int64_t) em_list[r0 + m] * ff + j] = from_f<T>(silu_f(to_f(from_f<T>(ag))) * to_f(from_f<T>(au)));
+            }
+        }
+    }
+}
+
+// per[(row, choice)][col] = Wd[expert][col] . hid[(row, choice)] (unweighted; exl3_mix_moe_combine adds the choices with their weights)
+template <typename T>
+__global__ __launch_bounds__(256) void moe_down_em_kernel(T* __restrict__ per, const T* __restrict__ hid, const T* __restrict__ wd, const int32_t* __restrict__ idx,
+                                                          int n_rows, int ff, int width)
+{
+    extern __shared__ int em_list[];
+    constexpr int VN = vecn<T>::N;
+    const int e = blockIdx.x, col = blockIdx.y * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+    const int cnt = em_list_rows(em_list, idx, n_rows, e);
+    if (cnt == 0 || col >= width) return;
+    const T* wr = wd + ((int64_t) e * width + col) * ff;
+    for (int r0 = blockIdx.z * EM_ROWS; r0 < cnt; r0 += gridDim.z * EM_ROWS)      // a long list is shared by the workgroups along z
+    {
+        float sa[EM_ROWS];
+        #pragma unroll
+        for (int m = 0; m < EM_ROWS; ++m) sa[m] = 0.f;
+        for (int c = lane * VN; c < ff; c += 64 * VN)
+        {
+            union { uint4 v; T e[VN]; } tw;
+            tw.v = *(const uint4*) (wr + c);
+            #pragma unroll
+            for (int m = 0; m < EM_ROWS; ++m)
+            {
+                if (r0 + m < cnt)
+                {
+                    union { uint4 v; T e[VN]; } tx;
+                    tx.v = *(const uint4*) (hid + (int64_t) em_list[r0 + m] * ff + c);
+                    #pragma unroll
+                    for (int q = 0; q < VN; ++q) sa[m] += to_f(tx.e[q]) * to_f(tw.e[q]);
+                }
+            }
+        }
+        #pragma unroll
+        for (int m = 0; m < EM_ROWS; ++m)
+        {
+            if (r0 + m < cnt)
+            {
+                const float a = wave_sum(sa[m]);
+                if (lane == 0) per[(int64_t) em_list[r0 + m] * width + col] = from_f<T>(a);
+            }
+        }
+    }
+}
+
+extern "C" int exl3_mix_moe_expert_major(void* per, void* hid, const void* h, const void* wg, const void* wu, const void* wd, const int32_t* idx,
+                                         int n, int top, int experts, int ff, int width, int dtype, void* stream)
+{
+    MIX_CHECK(per && hid && h && wg && wu && wd && idx && n >= 0 && top > 0 && experts > 0 && ff > 0 && width > 0, "mix_moe_expert_major: bad arguments");
+    const int vn = dtype == EXL3_MIX_BF16 ? 8 : 4;
+    MIX_CHECK(width % vn == 0 && ff % vn == 0 && (uintptr_t) h % 16 == 0 && (uintptr_t) wg % 16 == 0 && (uintptr_t) wu % 16 == 0 && (uintptr_t) wd % 16 == 0 &&
+              (uintptr_t) hid % 16 == 0, "mix_moe_expert_major: rows must be 16-byte aligned multiples of %d elements", vn);
+    MIX_CHECK((int64_t) n * top <= 8192, "mix_moe_expert_major: at most 8192 (row, choice) pairs");
+    if (n == 0) return EXL3_MIX_OK;
+    const int n_rows = n * top;
+    const size_t sm = (size_t) n_rows * sizeof(int);
+    const int gz = (n_rows + 2 * EM_ROWS - 1) / (2 * EM_ROWS);          // enough workgroups along z that a list of all rows is walked in two turns
+    MIX_DISPATCH_T(dtype, hipLaunchKernelGGL(moe_gate_up_em_kernel<T>, dim3(experts, (ff + 3) / 4, gz), dim3(256), sm, (hipStream_t) stream, (T*) hid, (const T*) h,
+                                             (const T*) wg, (const T*) wu, idx, n_rows, ff, width, top));
+    if (int rc = mix_check_launch("mix_moe_expert_major (gate, up)")) return rc;
+    MIX_DISPATCH_T(dtype, hipLaunchKernelGGL(moe_down_em_kernel<T>, dim3(experts, (width + 3) / 4, gz), dim3(256), sm, (hipStream_t) stream, (T*) per, (const T*) hid,
+                                             (const T*) wd, idx, n_rows, ff, width));
+    return mix_check_launch("mix_moe_expert_major (down)");
+}
+
 extern "C" int exl3_mix_silu_mul(void* out, const void* g, const void* u, int64_t count, int dtype, void* stream)
 {
     MIX_CHECK(out && g && u && count >= 0, "mix_silu_mul: bad arguments");

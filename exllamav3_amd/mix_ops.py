@@ -220,3 +220,28 @@ def moe_grouped(y, h, wg, wu, wd, idx, wts):
         torch.mm(hid[at: at + c], wd[e].t(), out=out[at: at + c])
         at += c
     _check(lib.exl3_mix_moe_combine(_p(y), _p(out), _p(where), _p(wts), n, top, width, code(h.dtype), _stream(h)))
+
+
+_identity: dict = {}
+
+
+def moe_expert_major(y, h, wg, wu, wd, idx, wts):
+    """Experts of a handful to a few dozen rows: each chosen expert's weights are streamed once for all its rows (no host read: capturable)."""
+    n, width = h.shape
+    experts, ff, _ = wg.shape
+    top = idx.shape[1]
+    _req(h.is_contiguous() and wg.is_contiguous() and wu.is_contiguous() and wd.is_contiguous() and y.is_contiguous() and y.dtype == h.dtype == wg.dtype, "moe_expert_major: layout")
+    _i32c(idx, "idx"); _f32c(wts, "wts")
+    hid = torch.empty((n * top, ff), dtype=h.dtype, device=h.device)
+    per = torch.empty((n * top, width), dtype=h.dtype, device=h.device)
+    key = (n * top, h.device)
+    if key not in _identity:
+        _identity[key] = torch.arange(n * top, dtype=torch.int32, device=h.device)
+    lib = _lib.mixlib()
+    _check(lib.exl3_mix_moe_expert_major(_p(per), _p(hid), _p(h), _p(wg), _p(wu), _p(wd), _p(idx), n, top, experts, ff, width, code(h.dtype), _stream(h)))
+    _check(lib.exl3_mix_moe_combine(_p(y), _p(per), _p(_identity[key]), _p(wts), n, top, width, code(h.dtype), _stream(h)))
+
+
+def moe_vector_layout(h, ff: int) -> bool:
+    vn = 8 if h.dtype == torch.bfloat16 else 4
+    return h.shape[1] % vn == 0 and ff % vn == 0

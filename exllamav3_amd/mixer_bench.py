@@ -109,7 +109,7 @@ def model_legs(size_name: str, prompt: int, ctx: int, steps: int, dev):
             def decode():
                 for s in slots[:bs]:
                     cache.length[s] = ctx
-                m.step(cache.begin_step([(s, [7]) for s in slots[:bs]]), cache)
+                m.step(cache.begin_step([(s, [7 + 101 * i]) for i, s in enumerate(slots[:bs])]), cache)       # different tokens: the rows route differently
             leg[f"decode_bs{bs}_ms_per_layer"] = _time(decode, steps) / reps * 1e3
         # the same batch-1 step as one captured graph (replayed at a fixed position): what the launches cost
         for s in slots[:1]:
@@ -209,6 +209,9 @@ def kernel_legs(size_name: str, prompt: int, ctx: int, dev):
 
         def moe():
             mix_ops.moe_gate_up(hid, hh, wg, wu, idx); mix_ops.moe_down(yy, hid, wd, idx, wt)
+        if bs > 1:
+            def moe():
+                mix_ops.moe_expert_major(yy, hh, wg, wu, wd, idx, wt)
         t = _time(moe, 50)
         by = min(bs * top, E) * 3 * eff * w * 2 if bs > 1 else top * 3 * eff * w * 2
         out[f"moe_decode_bs{bs}"] = {"us": t * 1e6, "GBps_distinct_weights": by / t / 1e9, "of_hbm": by / t / PEAK_HBM}

@@ -157,8 +157,10 @@ class PolyNormMLP:
 
 
 class SparseExperts:
-    # rows from which the expert-sorted matrix products take over from the weight-streaming kernels
+    # rows from which the expert-sorted matrix products take over from the weight-streaming kernels, and rows from which the streaming kernels
+    # walk each chosen expert once for all its rows instead of once per (row, choice)
     GROUPED_MIN_ROWS = 64
+    EXPERT_MAJOR_MIN_ROWS = 4
 
     def __init__(self, width: int, ff: int, experts: int, top: int):
         if not 0 < top <= experts:
@@ -183,6 +185,8 @@ class SparseExperts:
         y = torch.empty((sb.n, self.width), dtype=self.dtype, device=h.device)
         if sb.n >= self.GROUPED_MIN_ROWS:
             mix_ops.moe_grouped(y, h, self.w_gate, self.w_up, self.w_down, idx, wts)
+        elif sb.n >= self.EXPERT_MAJOR_MIN_ROWS and mix_ops.moe_vector_layout(h, self.ff):
+            mix_ops.moe_expert_major(y, h, self.w_gate, self.w_up, self.w_down, idx, wts)
         else:
             hid = torch.empty((sb.n * self.top, self.ff), dtype=self.dtype, device=h.device)
             mix_ops.moe_gate_up(hid, h, self.w_gate, self.w_up, idx)

@@ -112,6 +112,12 @@ int exl3_mix_moe_gate_up(void* hid, const void* h, const void* wg, const void* w
 int exl3_mix_moe_down(void* y, const void* hid, const void* wd, const int32_t* idx, const float* wts, int n, int top, int experts, int ff, int width,
                       int dtype, void* stream);
 
+/* Experts of a handful to a few dozen rows, expert-major: every expert's weights are streamed once for all the rows that chose it.
+ * hid [n*top][ff] (scratch), per [n*top][width] = the unweighted expert outputs per (row, choice); exl3_mix_moe_combine with where[i] = i adds the
+ * choices with their weights.  Rows must be 16-byte aligned multiples of 8 (bfloat16) / 4 (float32) elements. */
+int exl3_mix_moe_expert_major(void* per, void* hid, const void* h, const void* wg, const void* wu, const void* wd, const int32_t* idx,
+                              int n, int top, int experts, int ff, int width, int dtype, void* stream);
+
 /* Experts of many rows run as vendor matrix products over rows sorted by expert; these two kernels sit between and behind them:
  * out = silu(g) * u element by element, and y[n] = sum_r wts[n][r] * sorted[where[n*top + r]] (rows back in token order, weighted). */
 int exl3_mix_silu_mul(void* out, const void* g, const void* u, int64_t count, int dtype, void* stream);

@@ -201,7 +201,7 @@ def test_row_kernels_match_oracle(gpu, dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("n,E,top,ff,width", [(5, 6, 2, 40, 72), (70, 4, 1, 32, 64), (3, 3, 3, 20, 40), (150, 8, 3, 96, 128)])
+@pytest.mark.parametrize("n,E,top,ff,width", [(5, 6, 2, 40, 72), (70, 4, 1, 32, 64), (3, 3, 3, 20, 40), (150, 8, 3, 96, 128), (21, 8, 2, 64, 136), (40, 3, 2, 24, 48)])
 def test_router_and_experts_match_oracle(gpu, dtype, n, E, top, ff, width):
     from exllamav3_amd import mix_ops
     g = torch.Generator().manual_seed(n + E)
@@ -222,6 +222,10 @@ def test_router_and_experts_match_oracle(gpu, dtype, n, E, top, ff, width):
     mix_ops.moe_gate_up(hid, h.to(gpu), wg.to(gpu), wu.to(gpu), idx)
     mix_ops.moe_down(y, hid, wd.to(gpu), idx, wts)
     assert rel(y, ref) < TOL[dtype]
+    if mix_ops.moe_vector_layout(h, ff):
+        y3 = torch.full_like(y, float("nan"))
+        mix_ops.moe_expert_major(y3, h.to(gpu), wg.to(gpu), wu.to(gpu), wd.to(gpu), idx, wts)
+        assert rel(y3, ref) < TOL[dtype]
     if True:
         y2 = torch.empty_like(y)
         mix_ops.moe_grouped(y2, h.to(gpu), wg.to(gpu), wu.to(gpu), wd.to(gpu), idx, wts)
