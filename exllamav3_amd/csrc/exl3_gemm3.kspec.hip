@@ -206,7 +206,7 @@ void exl3_gemm3_kernel(const GemvArgs a)
     // weight ring: G3_NR slots of ONE decode step (4 tile rows) each, consumed round-robin by a loop that is unrolled G3_NR steps per trip, so every slot
     // is a fixed register set and every wait is countable: in front of step j exactly G3_NR - 1 younger ring loads are outstanding (round 4: the previous
     // two-block ring with its slot swap for odd block counts and the next chunk's activation rows requested across the loop made the compiler wait with
-    // vmcnt(0) at the loop head, i.e. for the refill issued a step earlier -- one full memory round trip exposed per trip: tools/isa_blocks.py, the reason
+    // vmcnt(0) at the loop head, i.e. for the refill issued a step earlier -- one full memory round trip exposed per trip, the reason
     // the 16-row pass ran at 45 % of its decode VALU bound)
     constexpr int NR = G3_NR;
     const int nsteps = 2 * nb;
