@@ -87,36 +87,39 @@ def test_attention_prefill_then_decode_matches_oracle(gpu, dtype, H, G, d, dv, W
         assert rel(out, want) < TOL[dtype], f"decode step {s}"
 
 
-def test_attention_window_edge_and_sink_show_in_the_output(gpu):
+@pytest.mark.parametrize("dtype,mfma", [(torch.float32, False), (torch.bfloat16, False), (torch.bfloat16, True)])
+def test_attention_window_edge_and_sink_show_in_the_output(gpu, dtype, mfma):
     """One key is made to dominate (its score is far above all others): just inside the window the output is that key's value, just outside it is not;
-    a huge sink takes the whole softmax mass and the output vanishes."""
+    a huge sink takes the whole softmax mass and the output vanishes.  Both prefill kernels and the decode kernel; the edge lies inside a key tile
+    of the matrix-core kernel for one row and on a tile border for another."""
     from exllamav3_amd import mix_ops
-    H = G = 1; d = dv = 16; W = 12; T = 40
+    d = dv = 16; T = 140
+    tol = 1e-4 if dtype == torch.float32 else 3e-2
     g = torch.Generator().manual_seed(3)
-    q = torch.randn(T, 1, d, generator=g) * 0.1; k = torch.randn(T, 1, d, generator=g) * 0.1; v = torch.randn(T, 1, dv, generator=g)
-    i = T - 1
-    for j, inside in ((i - W + 1, True), (i - W, False)):
-        kk = k.clone(); kk[j, 0] = q[i, 0] / q[i, 0].norm() ** 2 * 60.0            # score 60 * scale against scores ~0.01
-        cu, seq, pos, sl, p0, la = batch_tensors(gpu, [T])
-        ring_k = torch.zeros((1, W, 1, d), device=gpu); ring_v = torch.zeros((1, W, 1, dv), device=gpu)
-        vn = torch.empty((T, 1, dv), device=gpu)
-        mix_ops.attn_store(vn, ring_k, ring_v, kk.flatten(1).to(gpu), v.flatten(1).to(gpu), seq, pos, sl, la, 1e-5)
-        out = torch.empty((T, dv), device=gpu)
-        for sink, expect_zero in ((torch.full((1,), -30.0), False), (torch.full((1,), 200.0), True)):
-            mix_ops.attn_prefill(out, q.flatten(1).to(gpu), kk.flatten(1).to(gpu), vn, None, sink.to(gpu), cu, seq, pos, 1, 1.0, W)
-            o = out[i].cpu()
-            if expect_zero:
-                assert o.abs().max() < 1e-6
-            else:
-                hit = (o - vn[j, 0].cpu()).abs().max() < 1e-4
-                assert bool(hit) == inside
-            # the same row decoded against the ring (which holds positions T-W .. T-1)
-            mix_ops.attn_decode(out[:1], q[i].flatten().unsqueeze(0).to(gpu), ring_k, ring_v, None, sink.to(gpu), sl, la, 1, 1.0)
-            o = out[0].cpu()
-            if expect_zero:
-                assert o.abs().max() < 1e-6
-            else:
-                assert bool((o - vn[j, 0].cpu()).abs().max() < 1e-4) == inside
+    for W, i in ((12, T - 1), (76, T - 1), (64, 127)):                # row 139, window 76: first visible key 64 = a tile border; row 127, window 64: the same
+        q = (torch.randn(T, 1, d, generator=g) * 0.1).to(dtype); k = (torch.randn(T, 1, d, generator=g) * 0.1).to(dtype); v = torch.randn(T, 1, dv, generator=g).to(dtype)
+        for j, inside in ((i - W + 1, True), (i - W, False)):
+            kk = k.clone(); kk[j, 0] = (q[i, 0].float() / q[i, 0].float().norm() ** 2 * 60.0).to(dtype)            # score 60 against scores ~0.01
+            cu, seq, pos, sl, p0, la = batch_tensors(gpu, [i + 1])
+            ring_k = torch.zeros((1, W, 1, d), dtype=dtype, device=gpu); ring_v = torch.zeros((1, W, 1, dv), dtype=dtype, device=gpu)
+            n = i + 1
+            vn = torch.empty((n, 1, dv), dtype=dtype, device=gpu)
+            mix_ops.attn_store(vn, ring_k, ring_v, kk[:n].flatten(1).to(gpu), v[:n].flatten(1).to(gpu), seq, pos, sl, la, 1e-5)
+            out = torch.empty((n, dv), dtype=dtype, device=gpu)
+            for sink, expect_zero in ((torch.full((1,), -30.0), False), (torch.full((1,), 200.0), True)):
+                mix_ops.attn_prefill(out, q[:n].flatten(1).to(gpu), kk[:n].flatten(1).to(gpu), vn, None, sink.to(gpu), cu, seq, pos, 1, 1.0, W, max_rows=n, mfma=mfma)
+                o = out[i].float().cpu()
+                if expect_zero:
+                    assert o.abs().max() < 1e-6
+                else:
+                    assert bool((o - vn[j, 0].float().cpu()).abs().max() < tol) == inside, (W, i, j)
+                # the same row decoded against the ring (which holds the last W positions)
+                mix_ops.attn_decode(out[:1], q[i].flatten().unsqueeze(0).to(gpu), ring_k, ring_v, None, sink.to(gpu), sl, la, 1, 1.0)
+                o = out[0].float().cpu()
+                if expect_zero:
+                    assert o.abs().max() < 1e-6
+                else:
+                    assert bool((o - vn[j, 0].float().cpu()).abs().max() < tol) == inside, (W, i, j, "decode")
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
