@@ -476,3 +476,29 @@ def test_trace_replay_writes_the_same_logits_however_the_tokens_are_cut(models, 
     assert np.abs(np.concatenate([tog[0][1:], tog[6], tog[7]]) - whole[0]).max() < 1e-4
     refb = orc.forward(b).numpy()
     assert np.abs(tog[0][0] - refb[2]).max() < 1e-3 and np.abs(tog[5][0] - refb[7]).max() < 1e-3
+
+
+def test_a_cache_that_grows_under_captured_graphs_keeps_every_sequence(models):
+    """One job decodes alone from a one-slot cache until its decode step is a captured graph; then two more jobs arrive, the pool doubles twice (its
+    buffers move), the graphs are dropped and captured again -- and all three jobs still produce the oracle's greedy tokens."""
+    from exllamav3_amd.generator import Generator, Job
+    orc, ms, vocab = models["a"]
+    m = ms[torch.float32]
+    prompts = [toks(vocab, n, 90 + n) for n in (6, 3, 9)]
+    new = 14
+    want = []
+    for p in prompts:
+        s = list(p)
+        for _ in range(new):
+            s.append(int(orc.forward(s)[-1].argmax()))
+        want.append(s[len(p):])
+    gen = Generator(m, cache=m.new_cache(1), graphs=True)
+    jobs = [gen.enqueue(Job(list(prompts[0]), new))]
+    for _ in range(5):
+        gen.iterate()
+    assert gen.graph_replays >= 2 and gen.cache.capacity == 1
+    jobs += [gen.enqueue(Job(list(p), new)) for p in prompts[1:]]
+    while gen.busy():
+        gen.iterate()
+    assert gen.cache.capacity == 4
+    assert [j.output for j in jobs] == want
