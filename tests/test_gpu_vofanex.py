@@ -45,7 +45,7 @@ TOL = {torch.float32: 2e-5, torch.bfloat16: 3e-2}
 # ---- mechanisms alone -------------------------------------------------------------------------------------------------------
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("H,G,d,dv,W,lens", [(4, 2, 16, 24, 5, [17, 1, 9]), (3, 3, 40, 72, 64, [70]), (2, 1, 8, 8, 1, [6, 3]), (6, 2, 32, 130, 7, [20]), (2, 1, 96, 96, 37, [150, 66]), (1, 1, 136, 64, 100, [131]), (3, 1, 20, 12, 9, [40, 33])])
+@pytest.mark.parametrize("H,G,d,dv,W,lens", [(4, 2, 16, 24, 5, [17, 1, 9]), (3, 3, 40, 72, 64, [70]), (2, 1, 8, 8, 1, [6, 3]), (6, 2, 32, 130, 7, [20]), (2, 1, 96, 96, 37, [150, 66]), (1, 1, 136, 64, 100, [131]), (3, 1, 20, 12, 9, [40, 33]), (2, 1, 64, 64, 90, [300, 40]), (4, 2, 128, 128, 200, [530])])
 def test_attention_prefill_then_decode_matches_oracle(gpu, dtype, H, G, d, dv, W, lens):
     from exllamav3_amd import mix_ops
     g = torch.Generator().manual_seed(H * 100 + W)
