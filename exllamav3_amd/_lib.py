@@ -236,7 +236,7 @@ def _declare(l):
 # ---- the sequence-mixer library (include/exl3_mix.h, csrc/mix_*.hip) -------------------------------------------------------------
 MIX_LIB_PATH = os.path.join(_HERE, "libexl3_mix.so")
 MIX_HEADER_PATH = os.path.join(os.path.dirname(_HERE), "include", "exl3_mix.h")
-MIX_ABI_VERSION = 1
+MIX_ABI_VERSION = 2
 _mix = None
 
 
@@ -311,3 +311,16 @@ def _declare_mix(l):
     sig("exl3_mix_moe_combine", vp, vp, vp, vp, i32, i32, i32, i32, vp)
     sig("exl3_mix_attn_prefill_mfma", vp, vp, i64, vp, i64, vp, vp, i64, vp, vp, i32, i32, i32, i32, i32, i32, f32, i32, vp)
     sig("exl3_mix_moe_expert_major", vp, vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, vp)
+    sig("exl3_mix_moe_gate_up_act", vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, f32, i32, vp)
+    sig("exl3_mix_moe_expert_major_act", vp, vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, f32, i32, vp)
+    sig("exl3_mix_embed_copy", vp, vp, i64, vp, vp, i32, i32, i32, i32, vp)
+    sig("exl3_mix_residual_norm", vp, vp, i64, i32, vp, f32, i32, f32, vp, vp, vp, i64, i32, i32, i32, vp)
+    sig("exl3_mix_dyn_tanh_rows", vp, vp, vp, f32, vp, vp, i32, i32, i32, vp)
+    sig("exl3_mix_act", vp, vp, i64, i32, i32, i32, i32, vp)
+    sig("exl3_mix_glu_act", vp, vp, i64, vp, i64, i32, i32, i32, f32, i32, vp)
+    sig("exl3_mix_token_gate", vp, vp, i64, vp, i64, i32, vp, i32, i32, i32, i32, vp)
+    sig("exl3_mix_heads_gate", vp, vp, i64, i64, vp, i64, i32, i32, i32, i32, vp)
+    sig("exl3_mix_topk_sigmoid", vp, vp, vp, vp, f32, i32, i32, i32, i32, vp)
+    sig("exl3_mix_latent_prep", vp, vp, vp, i64, vp, vp, i64, vp, vp, vp, vp, vp, f32, f32, i32, i32, i32, i32, i32, i32, i32, i32, vp)
+    sig("exl3_mix_latent_fill_k", vp, i64, vp, i32, i32, i32, i32, i32, i32, vp)
+    sig("exl3_mix_latent_decode", vp, i64, i64, vp, i64, i64, vp, i64, vp, vp, vp, vp, i32, i32, i32, i32, i32, f32, i32, i32, vp)

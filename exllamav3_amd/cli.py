@@ -27,7 +27,7 @@ def _prepare(model_dir: str):
     from . import _lib, registry
     with open(os.path.join(model_dir, "config.json")) as f:
         arch = registry.architecture_of(json.load(f))
-    if arch == "Vofanex":
+    if registry.native_libraries(arch) == ("mix",):
         hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
         if os.path.exists(hipcc) or shutil.which("hipcc"):
             try:

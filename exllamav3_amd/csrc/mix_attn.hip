@@ -3,6 +3,7 @@
 // that starts from the sink.  The matrix-core prefill kernel for bfloat16 lives in mix_attn_mfma.hip; this file is the float32 path and
 // the decode path of both element types.
 #include "mix_common.cuh"
+#include "mix_attn_row.cuh"
 
 template <typename T>
 __global__ __launch_bounds__(64) void attn_store_kernel(T* __restrict__ v_norm, T* __restrict__ ring_k, T* __restrict__ ring_v, const T* __restrict__ k, int64_t k_ld,
@@ -35,122 +36,6 @@ __global__ __launch_bounds__(64) void attn_store_kernel(T* __restrict__ v_norm, 
     }
 }
 
-// One workgroup of AT_WAVES waves per (row, query head).  Keys kb + j * k_step, values vb + j * v_step, j < count: wave w takes the 64-key chunks
-// w, w + AT_WAVES, ... (one key per lane, its row read in 16-byte pieces when the layout allows), keeps its own running maximum, sum and
-// value accumulators (MAXV = ceil(vdim / 64) per lane), and the waves are merged through LDS at the end.  Wave 0 starts from the sink.
-#define AT_WAVES 4
-
-template <typename T> struct kvec;
-template <> struct kvec<bf16_t> { static constexpr int N = 8; };
-template <> struct kvec<float> { static constexpr int N = 4; };
-
-template <typename T, int MAXV>
-__device__ __forceinline__ void attn_row(T* __restrict__ out, const T* __restrict__ q, const T* __restrict__ kb, int64_t k_step, const T* __restrict__ vb,
-                                         int64_t v_step, int count, int dim, int vdim, float scale, bool has_sink, float sink, float gate, bool k_vec,
-                                         float* smem)
-{
-    float* qs = smem;                                   // [dim]
-    float* ps = qs + dim;                               // [AT_WAVES][64]
-    float* mg = ps + AT_WAVES * 64;                     // [AT_WAVES][2 + MAXV * 64]: m, l, accumulators
-    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
-    for (int i = threadIdx.x; i < dim; i += 64 * AT_WAVES) qs[i] = to_f(q[i]);
-    __syncthreads();
-    const bool seeded = has_sink && w == 0;
-    float m = seeded ? sink : -INFINITY, l = seeded ? 1.0f : 0.0f;
-    float acc[MAXV];
-    #pragma unroll
-    for (int i = 0; i < MAXV; ++i) acc[i] = 0.f;
-    float* pw = ps + w * 64;
-    constexpr int VN = kvec<T>::N;
-    for (int j0 = w * 64; j0 < count; j0 += 64 * AT_WAVES)
-    {
-        const int j = j0 + lane;
-        float s = -INFINITY;
-        if (j < count)
-        {
-            const T* kr = kb + (int64_t) j * k_step;
-            float d = 0.f;
-            if (k_vec)
-            {
-                for (int c = 0; c < dim; c += VN)
-                {
-                    union { uint4 v; T e[VN]; } t;
-                    t.v = *(const uint4*) (kr + c);
-                    #pragma unroll
-                    for (int e = 0; e < VN; ++e) d += qs[c + e] * to_f(t.e[e]);
-                }
-            }
-            else
-                for (int c = 0; c < dim; ++c) d += qs[c] * to_f(kr[c]);
-            s = d * scale;
-        }
-        const float m_new = fmaxf(m, wave_max(s));          // finite: j0 < count, so lane 0 of the chunk holds a score
-        const float p = (j < count) ? expf(s - m_new) : 0.f;
-        const float corr = expf(m - m_new);                 // m = -inf (nothing yet): 0
-        l = l * corr + wave_sum(p);
-        m = m_new;
-        pw[lane] = p;
-        __builtin_amdgcn_wave_barrier();                    // LDS serves a wave's accesses in order: its own stores are visible to the reads below
-        const int cnt = min(64, count - j0);
-        #pragma unroll
-        for (int i = 0; i < MAXV; ++i)
-        {
-            const int c = lane + 64 * i;
-            float a = acc[i] * corr;
-            if (c < vdim)
-            {
-                int jj = 0;
-                for (; jj + 8 <= cnt; jj += 8)                // eight value rows in flight, then the sums
-                {
-                    float vv[8];
-                    #pragma unroll
-                    for (int e = 0; e < 8; ++e) vv[e] = to_f(vb[(int64_t) (j0 + jj + e) * v_step + c]);
-                    #pragma unroll
-                    for (int e = 0; e < 8; ++e) a += pw[jj + e] * vv[e];
-                }
-                for (; jj < cnt; ++jj) a += pw[jj] * to_f(vb[(int64_t) (j0 + jj) * v_step + c]);
-            }
-            acc[i] = a;
-        }
-        __builtin_amdgcn_wave_barrier();
-    }
-    // merge the waves: wave 0 rescales every wave's partial to the common maximum
-    float* mine = mg + w * (2 + MAXV * 64);
-    if (lane == 0) { mine[0] = m; mine[1] = l; }
-    #pragma unroll
-    for (int i = 0; i < MAXV; ++i) mine[2 + i * 64 + lane] = acc[i];
-    __syncthreads();
-    if (w != 0) return;
-    float mt = -INFINITY;
-    #pragma unroll
-    for (int ww = 0; ww < AT_WAVES; ++ww) mt = fmaxf(mt, mg[ww * (2 + MAXV * 64)]);
-    float lt = 0.f;
-    #pragma unroll
-    for (int i = 0; i < MAXV; ++i) acc[i] = 0.f;
-    #pragma unroll
-    for (int ww = 0; ww < AT_WAVES; ++ww)
-    {
-        const float* o = mg + ww * (2 + MAXV * 64);
-        const float f = (o[0] == -INFINITY) ? 0.f : expf(o[0] - mt);
-        lt += o[1] * f;
-        #pragma unroll
-        for (int i = 0; i < MAXV; ++i) acc[i] += o[2 + i * 64 + lane] * f;
-    }
-    const float f = (lt > 0.f ? 1.0f / lt : 0.f) * gate;
-    #pragma unroll
-    for (int i = 0; i < MAXV; ++i)
-    {
-        const int c = lane + 64 * i;
-        if (c < vdim) out[c] = from_f<T>(acc[i] * f);
-    }
-}
-
-template <typename T>
-__device__ __forceinline__ bool rows_are_16_byte(const T* base, int64_t step, int dim)
-{
-    return ((uintptr_t) base % 16 == 0) && ((step * (int64_t) sizeof(T)) % 16 == 0) && (dim % kvec<T>::N == 0);
-}
-
 template <typename T, int MAXV>
 __global__ __launch_bounds__(64 * AT_WAVES) void attn_prefill_kernel(T* __restrict__ out, const T* __restrict__ q, int64_t q_ld, const T* __restrict__ k, int64_t k_ld,
                                                           const T* __restrict__ v_norm, const T* __restrict__ gate, int64_t gate_ld, const float* __restrict__ sink,
@@ -165,7 +50,7 @@ __global__ __launch_bounds__(64 * AT_WAVES) void attn_prefill_kernel(T* __restri
     const int lo = max(0, i - window + 1);
     const float gt = gate ? sigmoid_f(to_f(gate[(int64_t) n * gate_ld + h])) : 1.0f;
     const T* kb = k + (int64_t) (first + lo) * k_ld + (int64_t) g * dim;
-    attn_row<T, MAXV>(out + ((int64_t) n * heads + h) * vdim, q + (int64_t) n * q_ld + (int64_t) h * dim, kb, k_ld,
+    attn_row<T, MAXV>(out + ((int64_t) n * heads + h) * vdim, q + (int64_t) n * q_ld + (int64_t) h * dim, q, dim, kb, k_ld,
                       v_norm + ((int64_t) (first + lo) * kv_heads + g) * vdim, (int64_t) kv_heads * vdim,
                       i - lo + 1, dim, vdim, scale, sink != nullptr, sink ? sink[h] : 0.f, gt, rows_are_16_byte(kb, k_ld, dim), smem);
 }
@@ -183,7 +68,7 @@ __global__ __launch_bounds__(64 * AT_WAVES) void attn_decode_kernel(T* __restric
     const int64_t base = (int64_t) slots[n] * window * kv_heads + g;
     const float gt = gate ? sigmoid_f(to_f(gate[(int64_t) n * gate_ld + h])) : 1.0f;
     const T* kb = ring_k + base * dim;
-    attn_row<T, MAXV>(out + ((int64_t) n * heads + h) * vdim, q + (int64_t) n * q_ld + (int64_t) h * dim,
+    attn_row<T, MAXV>(out + ((int64_t) n * heads + h) * vdim, q + (int64_t) n * q_ld + (int64_t) h * dim, q, dim,
                       kb, (int64_t) kv_heads * dim, ring_v + base * vdim, (int64_t) kv_heads * vdim,
                       count, dim, vdim, scale, sink != nullptr, sink ? sink[h] : 0.f, gt, rows_are_16_byte(kb, (int64_t) kv_heads * dim, dim), smem);
 }

@@ -51,6 +51,15 @@ __device__ __forceinline__ float block_sum(float v, float* red)
 
 __device__ __forceinline__ float sigmoid_f(float z) { return 1.0f / (1.0f + expf(-z)); }
 __device__ __forceinline__ float silu_f(float z) { return z / (1.0f + expf(-z)); }
+// gated activations of two projections (g: gate, u: up).  EXL3_MIX_GLU_SILU: silu(g) u.  EXL3_MIX_GLU_CLAMPED_SWISH: g' = min(g, limit),
+// u' = clamp(u, -limit, limit), g' sigmoid(1.702 g') (u' + 1).
+__device__ __forceinline__ float glu_act_f(float g, float u, int kind, float limit)
+{
+    if (kind == EXL3_MIX_GLU_SILU) return silu_f(g) * u;
+    g = fminf(g, limit);
+    u = fminf(fmaxf(u, -limit), limit);
+    return g * sigmoid_f(1.702f * g) * (u + 1.0f);
+}
 // log(sigmoid(z)) without cancellation on either side
 __device__ __forceinline__ float log_sigmoid_f(float z) { return fminf(z, 0.f) - log1pf(expf(-fabsf(z))); }
 

@@ -45,7 +45,7 @@ __device__ __forceinline__ void dot_rows(const T* __restrict__ x, const T* __res
 
 template <typename T>
 __global__ __launch_bounds__(256) void moe_gate_up_kernel(T* __restrict__ hid, const T* __restrict__ h, const T* __restrict__ wg, const T* __restrict__ wu,
-                                                          const int32_t* __restrict__ idx, int experts, int ff, int width, int top, int vec)
+                                                          const int32_t* __restrict__ idx, int experts, int ff, int width, int top, int vec, int act, float limit)
 {
     const int row = blockIdx.x;                              // n * top + r
     const int j = blockIdx.y * 4 + (threadIdx.x >> 6);
@@ -59,7 +59,7 @@ __global__ __launch_bounds__(256) void moe_gate_up_kernel(T* __restrict__ hid, c
     float ag, au;
     dot_rows<T, true>(x, g, u, width, vec != 0, ag, au);
     // the two projections leave the matrix product in the activation type before the activation, like any other linear of the model
-    if (lane == 0) hid[(int64_t) row * ff + j] = from_f<T>(silu_f(to_f(from_f<T>(ag))) * to_f(from_f<T>(au)));
+    if (lane == 0) hid[(int64_t) row * ff + j] = from_f<T>(glu_act_f(to_f(from_f<T>(ag)), to_f(from_f<T>(au)), act, limit));
 }
 
 template <typename T>
@@ -134,7 +134,7 @@ __device__ __forceinline__ int em_list_rows(int* list, const int32_t* __restrict
 
 template <typename T>
 __global__ __launch_bounds__(256) void moe_gate_up_em_kernel(T* __restrict__ hid, const T* __restrict__ h, const T* __restrict__ wg, const T* __restrict__ wu,
-                                                             const int32_t* __restrict__ idx, int n_rows, int ff, int width, int top)
+                                                             const int32_t* __restrict__ idx, int n_rows, int ff, int width, int top, int act, float limit)
 {
     extern __shared__ int em_list[];
     constexpr int VN = vecn<T>::N;
@@ -174,7 +174,7 @@ __global__ __launch_bounds__(256) void moe_gate_up_em_kernel(T* __restrict__ hid
             if (r0 + m < cnt)
             {
                 const float ag = wave_sum(sa[m]), au = wave_sum(sb[m]);
-                if (lane == 0) hid[(int64_t) em_list[r0 + m] * ff + j] = from_f<T>(silu_f(to_f(from_f<T>(ag))) * to_f(from_f<T>(au)));
+                if (lane == 0) hid[(int64_t) em_list[r0 + m] * ff + j] = from_f<T>(glu_act_f(to_f(from_f<T>(ag)), to_f(from_f<T>(au)), act, limit));
             }
         }
     }
@@ -224,9 +224,10 @@ __global__ __launch_bounds__(256) void moe_down_em_kernel(T* __restrict__ per, c
     }
 }
 
-extern "C" int exl3_mix_moe_expert_major(void* per, void* hid, const void* h, const void* wg, const void* wu, const void* wd, const int32_t* idx,
-                                         int n, int top, int experts, int ff, int width, int dtype, void* stream)
+extern "C" int exl3_mix_moe_expert_major_act(void* per, void* hid, const void* h, const void* wg, const void* wu, const void* wd, const int32_t* idx,
+                                             int n, int top, int experts, int ff, int width, int act, float limit, int dtype, void* stream)
 {
+    MIX_CHECK(act == EXL3_MIX_GLU_SILU || act == EXL3_MIX_GLU_CLAMPED_SWISH, "mix_moe_expert_major: unknown activation %d", act);
     MIX_CHECK(per && hid && h && wg && wu && wd && idx && n >= 0 && top > 0 && experts > 0 && ff > 0 && width > 0, "mix_moe_expert_major: bad arguments");
     const int vn = dtype == EXL3_MIX_BF16 ? 8 : 4;
     MIX_CHECK(width % vn == 0 && ff % vn == 0 && (uintptr_t) h % 16 == 0 && (uintptr_t) wg % 16 == 0 && (uintptr_t) wu % 16 == 0 && (uintptr_t) wd % 16 == 0 &&
@@ -237,11 +238,17 @@ extern "C" int exl3_mix_moe_expert_major(void* per, void* hid, const void* h, co
     const size_t sm = (size_t) n_rows * sizeof(int);
     const int gz = (n_rows + 2 * EM_ROWS - 1) / (2 * EM_ROWS);          // enough workgroups along z that a list of all rows is walked in two turns
     MIX_DISPATCH_T(dtype, hipLaunchKernelGGL(moe_gate_up_em_kernel<T>, dim3(experts, (ff + 3) / 4, gz), dim3(256), sm, (hipStream_t) stream, (T*) hid, (const T*) h,
-                                             (const T*) wg, (const T*) wu, idx, n_rows, ff, width, top));
+                                             (const T*) wg, (const T*) wu, idx, n_rows, ff, width, top, act, limit));
     if (int rc = mix_check_launch("mix_moe_expert_major (gate, up)")) return rc;
     MIX_DISPATCH_T(dtype, hipLaunchKernelGGL(moe_down_em_kernel<T>, dim3(experts, (width + 3) / 4, gz), dim3(256), sm, (hipStream_t) stream, (T*) per, (const T*) hid,
                                              (const T*) wd, idx, n_rows, ff, width));
     return mix_check_launch("mix_moe_expert_major (down)");
+}
+
+extern "C" int exl3_mix_moe_expert_major(void* per, void* hid, const void* h, const void* wg, const void* wu, const void* wd, const int32_t* idx,
+                                         int n, int top, int experts, int ff, int width, int dtype, void* stream)
+{
+    return exl3_mix_moe_expert_major_act(per, hid, h, wg, wu, wd, idx, n, top, experts, ff, width, EXL3_MIX_GLU_SILU, 0.f, dtype, stream);
 }
 
 extern "C" int exl3_mix_silu_mul(void* out, const void* g, const void* u, int64_t count, int dtype, void* stream)
@@ -261,16 +268,23 @@ extern "C" int exl3_mix_moe_combine(void* y, const void* sorted, const int32_t* 
     return mix_check_launch("mix_moe_combine");
 }
 
-extern "C" int exl3_mix_moe_gate_up(void* hid, const void* h, const void* wg, const void* wu, const int32_t* idx, int n, int top, int experts, int ff, int width,
-                                    int dtype, void* stream)
+extern "C" int exl3_mix_moe_gate_up_act(void* hid, const void* h, const void* wg, const void* wu, const int32_t* idx, int n, int top, int experts, int ff, int width,
+                                        int act, float limit, int dtype, void* stream)
 {
+    MIX_CHECK(act == EXL3_MIX_GLU_SILU || act == EXL3_MIX_GLU_CLAMPED_SWISH, "mix_moe_gate_up: unknown activation %d", act);
     MIX_CHECK(hid && h && wg && wu && idx && n >= 0 && top > 0 && experts > 0 && ff > 0 && width > 0, "mix_moe_gate_up: bad arguments");
     if (n == 0) return EXL3_MIX_OK;
     const int vn = dtype == EXL3_MIX_BF16 ? 8 : 4;
     const int vec = width % vn == 0 && (uintptr_t) h % 16 == 0 && (uintptr_t) wg % 16 == 0 && (uintptr_t) wu % 16 == 0;
     MIX_DISPATCH_T(dtype, hipLaunchKernelGGL(moe_gate_up_kernel<T>, dim3(n * top, (ff + 3) / 4), dim3(256), 0, (hipStream_t) stream, (T*) hid, (const T*) h,
-                                             (const T*) wg, (const T*) wu, idx, experts, ff, width, top, vec));
+                                             (const T*) wg, (const T*) wu, idx, experts, ff, width, top, vec, act, limit));
     return mix_check_launch("mix_moe_gate_up");
+}
+
+extern "C" int exl3_mix_moe_gate_up(void* hid, const void* h, const void* wg, const void* wu, const int32_t* idx, int n, int top, int experts, int ff, int width,
+                                    int dtype, void* stream)
+{
+    return exl3_mix_moe_gate_up_act(hid, h, wg, wu, idx, n, top, experts, ff, width, EXL3_MIX_GLU_SILU, 0.f, dtype, stream);
 }
 
 extern "C" int exl3_mix_moe_down(void* y, const void* hid, const void* wd, const int32_t* idx, const float* wts, int n, int top, int experts, int ff, int width,

@@ -1,0 +1,232 @@
+// Row-wise kernels of pre-norm blocks over a float32 residual stream whose norm needs no statistics (Dynamic Tanh), and the small pieces
+// between their matrix products: the embedding with a copy in the activation type, the residual update (plain or with the addend divided by
+// its root mean square) fused with what the next consumer reads (the next norm, or the stream in the activation type), the last norm on chosen
+// rows, element-wise activations (plain and gated, with clamps), a per-token gate from an embedding table, a gate applied across a
+// head-major layout, and a router with sigmoid scores.  Sums and the residual are float32.
+#include "mix_common.cuh"
+
+#define ROW_THREADS 256
+#define ROW_WAVES 4
+
+__device__ __forceinline__ float gelu_tanh_f(float z) { return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z))); }
+
+template <typename T>
+__global__ __launch_bounds__(ROW_THREADS) void embed_copy_kernel(float* __restrict__ x, T* __restrict__ xc, int64_t xc_ld, const T* __restrict__ table,
+                                                                 const int32_t* __restrict__ tokens, int width, int vocab)
+{
+    const int n = blockIdx.x;
+    int tok = tokens[n];
+    tok = tok < 0 ? 0 : (tok >= vocab ? vocab - 1 : tok);
+    const T* src = table + (int64_t) tok * width;
+    for (int i = threadIdx.x; i < width; i += ROW_THREADS)
+    {
+        const T v = src[i];
+        x[(int64_t) n * width + i] = to_f(v);
+        if (xc) xc[(int64_t) n * xc_ld + i] = v;
+    }
+}
+
+// mode 0: x stays; 1: x += y'; 2: x = y'   with y' = y, or y / rms(y) * rms_w when rms_w is given.
+// out 0: nothing; 1: h = x in the activation type; 2: h = tanh(alpha x) w + b.
+template <typename T>
+__global__ __launch_bounds__(ROW_THREADS) void residual_norm_kernel(float* __restrict__ x, const T* __restrict__ y, int64_t y_ld, int mode, const float* __restrict__ rms_w,
+                                                                    float eps, int out, float alpha, const float* __restrict__ w, const float* __restrict__ b,
+                                                                    T* __restrict__ h, int64_t h_ld, int width)
+{
+    __shared__ float red[ROW_WAVES];
+    const int n = blockIdx.x;
+    float* xr = x + (int64_t) n * width;
+    const T* yr = y + (int64_t) n * y_ld;
+    float inv = 1.0f;
+    if (mode != 0 && rms_w)
+    {
+        float ss = 0.f;
+        for (int i = threadIdx.x; i < width; i += ROW_THREADS) { const float v = to_f(yr[i]); ss += v * v; }
+        ss = block_sum<ROW_WAVES>(ss, red);
+        inv = 1.0f / sqrtf(ss / (float) width + eps);
+    }
+    T* hr = h + (int64_t) n * h_ld;
+    for (int i = threadIdx.x; i < width; i += ROW_THREADS)
+    {
+        float v = xr[i];
+        if (mode != 0)
+        {
+            float a = to_f(yr[i]);
+            if (rms_w) a = a * inv * rms_w[i];
+            v = mode == 1 ? v + a : a;
+            xr[i] = v;
+        }
+        if (out == 1) hr[i] = from_f<T>(v);
+        else if (out == 2) hr[i] = from_f<T>(tanhf(alpha * v) * w[i] + b[i]);
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(ROW_THREADS) void dyn_tanh_rows_kernel(T* __restrict__ h, const float* __restrict__ x, const int32_t* __restrict__ rows, float alpha,
+                                                                    const float* __restrict__ w, const float* __restrict__ b, int width)
+{
+    const int n = blockIdx.x;
+    const float* xr = x + (int64_t) (rows ? rows[n] : n) * width;
+    for (int i = threadIdx.x; i < width; i += ROW_THREADS) h[(int64_t) n * width + i] = from_f<T>(tanhf(alpha * xr[i]) * w[i] + b[i]);
+}
+
+// plain activations: 0 = relu(z)^2, 1 = gelu (tanh form), 2 = silu
+template <typename T>
+__global__ __launch_bounds__(256) void act_kernel(T* __restrict__ out, const T* __restrict__ z, int64_t z_ld, int ff, int kind)
+{
+    const int n = blockIdx.y;
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= ff) return;
+    const float v = to_f(z[(int64_t) n * z_ld + i]);
+    float r;
+    if (kind == 0) { const float t = fmaxf(v, 0.f); r = t * t; }
+    else if (kind == 1) r = gelu_tanh_f(v);
+    else r = silu_f(v);
+    out[(int64_t) n * ff + i] = from_f<T>(r);
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void glu_act_kernel(T* __restrict__ out, const T* __restrict__ g, int64_t g_ld, const T* __restrict__ u, int64_t u_ld, int ff, int kind, float limit)
+{
+    const int n = blockIdx.y;
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= ff) return;
+    out[(int64_t) n * ff + i] = from_f<T>(glu_act_f(to_f(g[(int64_t) n * g_ld + i]), to_f(u[(int64_t) n * u_ld + i]), kind, limit));
+}
+
+// out[n][j] = gelu_tanh(gate[n][j]) * table[tokens[n]][col0 + j]
+template <typename T>
+__global__ __launch_bounds__(64) void token_gate_kernel(T* __restrict__ out, const T* __restrict__ gate, int64_t gate_ld, const T* __restrict__ table, int64_t table_ld,
+                                                        int col0, const int32_t* __restrict__ tokens, int dim, int vocab)
+{
+    const int n = blockIdx.x;
+    int tok = tokens[n];
+    tok = tok < 0 ? 0 : (tok >= vocab ? vocab - 1 : tok);
+    const T* e = table + (int64_t) tok * table_ld + col0;
+    for (int j = threadIdx.x; j < dim; j += 64)
+        out[(int64_t) n * dim + j] = from_f<T>(gelu_tanh_f(to_f(gate[(int64_t) n * gate_ld + j])) * to_f(e[j]));
+}
+
+// out[n][h * vdim + v] = a[n * a_row + h * a_head + v] * (gate ? sigmoid(gate[n][h * vdim + v]) : 1)
+template <typename T>
+__global__ __launch_bounds__(256) void heads_gate_kernel(T* __restrict__ out, const T* __restrict__ a, int64_t a_row, int64_t a_head, const T* __restrict__ gate,
+                                                         int64_t gate_ld, int heads, int vdim)
+{
+    const int n = blockIdx.x;
+    for (int t = threadIdx.x; t < heads * vdim; t += 256)
+    {
+        const int h = t / vdim, v = t - h * vdim;
+        float r = to_f(a[(int64_t) n * a_row + (int64_t) h * a_head + v]);
+        if (gate) r *= sigmoid_f(to_f(gate[(int64_t) n * gate_ld + t]));
+        out[(int64_t) n * heads * vdim + t] = from_f<T>(r);
+    }
+}
+
+// Router with independent scores: s = sigmoid(z); the `top` experts with the largest s + correction are chosen (ties go to the lower index), and
+// their weights are s / (sum of the chosen s + 1e-20) * scale (normalise = 0: s * scale).
+__global__ void topk_sigmoid_kernel(int32_t* __restrict__ idx, float* __restrict__ wts, const float* __restrict__ logits, const float* __restrict__ correction,
+                                    float scale, int normalise, int n, int experts, int top)
+{
+    const int t = blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= n) return;
+    const float* l = logits + (int64_t) t * experts;
+    int32_t* id = idx + (int64_t) t * top;
+    float* w = wts + (int64_t) t * top;
+    float sum = 0.f;
+    for (int r = 0; r < top; ++r)
+    {
+        int best = -1; float bv = 0.f, bs = 0.f;
+        for (int e = 0; e < experts; ++e)
+        {
+            bool taken = false;
+            for (int p = 0; p < r; ++p) taken |= (id[p] == e);
+            if (taken) continue;
+            const float s = sigmoid_f(l[e]);
+            const float v = correction ? s + correction[e] : s;
+            if (best < 0 || v > bv) { best = e; bv = v; bs = s; }
+        }
+        id[r] = best; w[r] = bs; sum += bs;
+    }
+    const float f = normalise ? scale / (sum + 1e-20f) : scale;
+    for (int r = 0; r < top; ++r) w[r] = w[r] * f;
+}
+
+extern "C" int exl3_mix_embed_copy(float* x, void* xc, int64_t xc_ld, const void* table, const int32_t* tokens, int n, int width, int vocab, int dtype, void* stream)
+{
+    MIX_CHECK(x && table && tokens && n >= 0 && width > 0 && vocab > 0 && (!xc || xc_ld >= width), "mix_embed_copy: bad arguments");
+    if (n == 0) return EXL3_MIX_OK;
+    MIX_DISPATCH_T(dtype, hipLaunchKernelGGL(embed_copy_kernel<T>, dim3(n), dim3(ROW_THREADS), 0, (hipStream_t) stream, x, (T*) xc, xc_ld, (const T*) table, tokens, width, vocab));
+    return mix_check_launch("mix_embed_copy");
+}
+
+extern "C" int exl3_mix_residual_norm(float* x, const void* y, int64_t y_ld, int mode, const float* rms_w, float eps, int out, float alpha, const float* w, const float* b,
+                                      void* h, int64_t h_ld, int n, int width, int dtype, void* stream)
+{
+    MIX_CHECK(x && n >= 0 && width > 0 && mode >= 0 && mode <= 2 && out >= 0 && out <= 2, "mix_residual_norm: bad arguments");
+    MIX_CHECK(mode == 0 || (y && y_ld >= width), "mix_residual_norm: an addend is needed");
+    MIX_CHECK(out == 0 || (h && h_ld >= width), "mix_residual_norm: an output is needed");
+    MIX_CHECK(out != 2 || (w && b), "mix_residual_norm: the norm needs its weight and bias");
+    if (n == 0 || (mode == 0 && out == 0)) return EXL3_MIX_OK;
+    MIX_DISPATCH_T(dtype, hipLaunchKernelGGL(residual_norm_kernel<T>, dim3(n), dim3(ROW_THREADS), 0, (hipStream_t) stream, x, (const T*) y, y_ld, mode, rms_w, eps, out, alpha,
+                                             w, b, (T*) h, h_ld, width));
+    return mix_check_launch("mix_residual_norm");
+}
+
+extern "C" int exl3_mix_dyn_tanh_rows(void* h, const float* x, const int32_t* rows, float alpha, const float* w, const float* b, int n, int width, int dtype, void* stream)
+{
+    MIX_CHECK(h && x && w && b && n >= 0 && width > 0, "mix_dyn_tanh_rows: bad arguments");
+    if (n == 0) return EXL3_MIX_OK;
+    MIX_DISPATCH_T(dtype, hipLaunchKernelGGL(dyn_tanh_rows_kernel<T>, dim3(n), dim3(ROW_THREADS), 0, (hipStream_t) stream, (T*) h, x, rows, alpha, w, b, width));
+    return mix_check_launch("mix_dyn_tanh_rows");
+}
+
+extern "C" int exl3_mix_act(void* out, const void* z, int64_t z_ld, int n, int ff, int kind, int dtype, void* stream)
+{
+    MIX_CHECK(out && z && n >= 0 && n <= 65535 * 1024 && ff > 0 && z_ld >= ff && kind >= 0 && kind <= 2, "mix_act: bad arguments");
+    for (int r0 = 0; r0 < n; r0 += 65535)
+    {
+        const int rows = n - r0 < 65535 ? n - r0 : 65535;
+        MIX_DISPATCH_T(dtype, hipLaunchKernelGGL(act_kernel<T>, dim3((ff + 255) / 256, rows), dim3(256), 0, (hipStream_t) stream, (T*) out + (int64_t) r0 * ff,
+                                                 (const T*) z + (int64_t) r0 * z_ld, z_ld, ff, kind));
+    }
+    return mix_check_launch("mix_act");
+}
+
+extern "C" int exl3_mix_glu_act(void* out, const void* g, int64_t g_ld, const void* u, int64_t u_ld, int n, int ff, int kind, float limit, int dtype, void* stream)
+{
+    MIX_CHECK(out && g && u && n >= 0 && ff > 0 && g_ld >= ff && u_ld >= ff && kind >= 0 && kind <= 1, "mix_glu_act: bad arguments");
+    for (int r0 = 0; r0 < n; r0 += 65535)
+    {
+        const int rows = n - r0 < 65535 ? n - r0 : 65535;
+        MIX_DISPATCH_T(dtype, hipLaunchKernelGGL(glu_act_kernel<T>, dim3((ff + 255) / 256, rows), dim3(256), 0, (hipStream_t) stream, (T*) out + (int64_t) r0 * ff,
+                                                 (const T*) g + (int64_t) r0 * g_ld, g_ld, (const T*) u + (int64_t) r0 * u_ld, u_ld, ff, kind, limit));
+    }
+    return mix_check_launch("mix_glu_act");
+}
+
+extern "C" int exl3_mix_token_gate(void* out, const void* gate, int64_t gate_ld, const void* table, int64_t table_ld, int col0, const int32_t* tokens,
+                                   int n, int dim, int vocab, int dtype, void* stream)
+{
+    MIX_CHECK(out && gate && table && tokens && n >= 0 && dim > 0 && vocab > 0 && gate_ld >= dim && col0 >= 0 && table_ld >= col0 + dim, "mix_token_gate: bad arguments");
+    if (n == 0) return EXL3_MIX_OK;
+    MIX_DISPATCH_T(dtype, hipLaunchKernelGGL(token_gate_kernel<T>, dim3(n), dim3(64), 0, (hipStream_t) stream, (T*) out, (const T*) gate, gate_ld, (const T*) table, table_ld,
+                                             col0, tokens, dim, vocab));
+    return mix_check_launch("mix_token_gate");
+}
+
+extern "C" int exl3_mix_heads_gate(void* out, const void* a, int64_t a_row, int64_t a_head, const void* gate, int64_t gate_ld, int n, int heads, int vdim, int dtype, void* stream)
+{
+    MIX_CHECK(out && a && n >= 0 && heads > 0 && vdim > 0 && (!gate || gate_ld >= (int64_t) heads * vdim), "mix_heads_gate: bad arguments");
+    if (n == 0) return EXL3_MIX_OK;
+    MIX_DISPATCH_T(dtype, hipLaunchKernelGGL(heads_gate_kernel<T>, dim3(n), dim3(256), 0, (hipStream_t) stream, (T*) out, (const T*) a, a_row, a_head, (const T*) gate, gate_ld,
+                                             heads, vdim));
+    return mix_check_launch("mix_heads_gate");
+}
+
+extern "C" int exl3_mix_topk_sigmoid(int32_t* idx, float* wts, const float* logits, const float* correction, float scale, int normalise, int n, int experts, int top, void* stream)
+{
+    MIX_CHECK(idx && wts && logits && n >= 0 && experts > 0 && top > 0 && top <= experts, "mix_topk_sigmoid: bad arguments (top %d of %d)", top, experts);
+    if (n == 0) return EXL3_MIX_OK;
+    hipLaunchKernelGGL(topk_sigmoid_kernel, dim3((n + 63) / 64), dim3(64), 0, (hipStream_t) stream, idx, wts, logits, correction, scale, normalise, n, experts, top);
+    return mix_check_launch("mix_topk_sigmoid");
+}

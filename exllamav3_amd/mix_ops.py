@@ -196,7 +196,7 @@ def moe_down(y, hid, wd, idx, wts):
     _check(_lib.mixlib().exl3_mix_moe_down(_p(y), _p(hid), _p(wd), _p(idx), _p(wts), n, top, experts, ff, width, code(y.dtype), _stream(y)))
 
 
-def moe_grouped(y, h, wg, wu, wd, idx, wts):
+def moe_grouped(y, h, wg, wu, wd, idx, wts, act_kind: int = 0, limit: float = 0.0):
     """Experts of many rows: rows sorted by expert (device), one host read of the per-expert counts, then per expert three vendor matrix products
     with the activation kernel between them, and the weighted un-sort.  Same result as moe_gate_up + moe_down up to rounding."""
     n, width = h.shape
@@ -216,7 +216,7 @@ def moe_grouped(y, h, wg, wu, wd, idx, wts):
             continue
         seg = xs[at: at + c]
         g, u = torch.nn.functional.linear(seg, wg[e]), torch.nn.functional.linear(seg, wu[e])
-        _check(lib.exl3_mix_silu_mul(_p(hid[at: at + c]), _p(g), _p(u), c * ff, code(h.dtype), _stream(h)))
+        _check(lib.exl3_mix_glu_act(_p(hid[at: at + c]), _p(g), ff, _p(u), ff, c, ff, act_kind, limit, code(h.dtype), _stream(h)))
         torch.mm(hid[at: at + c], wd[e].t(), out=out[at: at + c])
         at += c
     _check(lib.exl3_mix_moe_combine(_p(y), _p(out), _p(where), _p(wts), n, top, width, code(h.dtype), _stream(h)))
@@ -225,7 +225,7 @@ def moe_grouped(y, h, wg, wu, wd, idx, wts):
 _identity: dict = {}
 
 
-def moe_expert_major(y, h, wg, wu, wd, idx, wts):
+def moe_expert_major(y, h, wg, wu, wd, idx, wts, act_kind: int = 0, limit: float = 0.0):
     """Experts of a handful to a few dozen rows: each chosen expert's weights are streamed once for all its rows (no host read: capturable)."""
     n, width = h.shape
     experts, ff, _ = wg.shape
@@ -238,10 +238,145 @@ def moe_expert_major(y, h, wg, wu, wd, idx, wts):
     if key not in _identity:
         _identity[key] = torch.arange(n * top, dtype=torch.int32, device=h.device)
     lib = _lib.mixlib()
-    _check(lib.exl3_mix_moe_expert_major(_p(per), _p(hid), _p(h), _p(wg), _p(wu), _p(wd), _p(idx), n, top, experts, ff, width, code(h.dtype), _stream(h)))
+    _check(lib.exl3_mix_moe_expert_major_act(_p(per), _p(hid), _p(h), _p(wg), _p(wu), _p(wd), _p(idx), n, top, experts, ff, width, act_kind, limit, code(h.dtype), _stream(h)))
     _check(lib.exl3_mix_moe_combine(_p(y), _p(per), _p(_identity[key]), _p(wts), n, top, width, code(h.dtype), _stream(h)))
 
 
 def moe_vector_layout(h, ff: int) -> bool:
     vn = 8 if h.dtype == torch.bfloat16 else 4
     return h.shape[1] % vn == 0 and ff % vn == 0
+
+
+# ---- pre-norm blocks with a statistics-free norm, gated activations, sigmoid router (csrc/mix_rowops.hip) ------------------------------------------
+GLU_SILU, GLU_CLAMPED_SWISH = 0, 1
+ACT_RELU2, ACT_GELU_TANH, ACT_SILU = 0, 1, 2
+RES_KEEP, RES_ADD, RES_SET = 0, 1, 2
+OUT_NONE, OUT_CAST, OUT_DYN_TANH = 0, 1, 2
+
+
+def embed_copy(x: torch.Tensor, xc_view: torch.Tensor | None, table: torch.Tensor, tokens: torch.Tensor):
+    n, width = x.shape
+    _f32c(x, "x"); _i32c(tokens, "tokens")
+    _req(tokens.numel() == n and table.is_contiguous() and table.shape[1] == width, "embed_copy: shapes")
+    if xc_view is not None:
+        _req(xc_view.dtype == table.dtype and xc_view.shape[0] == n, "embed_copy: the copy has the table's element type")
+    _check(_lib.mixlib().exl3_mix_embed_copy(_p(x), _p(xc_view), 0 if xc_view is None else _view(xc_view, width, "xc"), _p(table), _p(tokens), n, width, table.shape[0],
+                                              code(table.dtype), _stream(x)))
+
+
+def residual_norm(x: torch.Tensor, y_view: torch.Tensor | None, mode: int, rms_w: torch.Tensor | None, eps: float, out: int, alpha: float, w: torch.Tensor | None,
+                  b: torch.Tensor | None, h_view: torch.Tensor | None):
+    """x (float32 residual, in place) = x | x + y' | y', y' = y or y / rms(y) * rms_w; h = nothing | x in the activation type | tanh(alpha x) w + b."""
+    n, width = x.shape
+    _f32c(x, "x")
+    ref = y_view if y_view is not None else h_view
+    _req(ref is not None, "residual_norm: nothing to do")
+    if mode != RES_KEEP:
+        _req(y_view is not None and y_view.shape[0] == n, "residual_norm: y")
+    if rms_w is not None:
+        _f32c(rms_w, "rms_w"); _req(rms_w.numel() == width, "residual_norm: rms_w")
+    if out != OUT_NONE:
+        _req(h_view is not None and h_view.shape[0] == n and h_view.dtype == ref.dtype, "residual_norm: h")
+    if out == OUT_DYN_TANH:
+        _f32c(w, "w"); _f32c(b, "b"); _req(w.numel() == width and b.numel() == width, "residual_norm: norm weight / bias")
+    _check(_lib.mixlib().exl3_mix_residual_norm(_p(x), _p(y_view) if mode != RES_KEEP else None, 0 if (y_view is None or mode == RES_KEEP) else _view(y_view, width, "y"), mode,
+                                                 _p(rms_w), eps, out, alpha, _p(w), _p(b), _p(h_view) if out != OUT_NONE else None,
+                                                 0 if (h_view is None or out == OUT_NONE) else _view(h_view, width, "h"), n, width, code(ref.dtype), _stream(x)))
+
+
+def dyn_tanh_rows(h: torch.Tensor, x: torch.Tensor, rows: torch.Tensor | None, alpha: float, w: torch.Tensor, b: torch.Tensor):
+    n, width = h.shape
+    _f32c(x, "x"); _f32c(w, "w"); _f32c(b, "b")
+    _req(h.is_contiguous() and x.shape[1] == width and w.numel() == width and b.numel() == width, "dyn_tanh_rows: shapes")
+    if rows is not None:
+        _i32c(rows, "rows"); _req(rows.numel() == n, "dyn_tanh_rows: rows")
+    else:
+        _req(x.shape[0] == n, "dyn_tanh_rows: rows of x")
+    _check(_lib.mixlib().exl3_mix_dyn_tanh_rows(_p(h), _p(x), _p(rows), alpha, _p(w), _p(b), n, width, code(h.dtype), _stream(x)))
+
+
+def act(out: torch.Tensor, z_view: torch.Tensor, kind: int):
+    n, ff = out.shape
+    _req(out.is_contiguous() and z_view.dtype == out.dtype and z_view.shape[0] == n, "act: shapes")
+    _check(_lib.mixlib().exl3_mix_act(_p(out), _p(z_view), _view(z_view, ff, "z"), n, ff, kind, code(out.dtype), _stream(out)))
+
+
+def glu_act(out: torch.Tensor, g_view: torch.Tensor, u_view: torch.Tensor, kind: int, limit: float = 0.0):
+    n, ff = out.shape
+    _req(out.is_contiguous() and g_view.dtype == out.dtype == u_view.dtype and g_view.shape[0] == n and u_view.shape[0] == n, "glu_act: shapes")
+    _check(_lib.mixlib().exl3_mix_glu_act(_p(out), _p(g_view), _view(g_view, ff, "g"), _p(u_view), _view(u_view, ff, "u"), n, ff, kind, limit, code(out.dtype), _stream(out)))
+
+
+def token_gate(out: torch.Tensor, gate_view: torch.Tensor, table: torch.Tensor, col0: int, tokens: torch.Tensor):
+    n, dim = out.shape
+    _i32c(tokens, "tokens")
+    _req(out.is_contiguous() and gate_view.dtype == out.dtype == table.dtype and table.is_contiguous() and table.dim() == 2 and tokens.numel() == n
+         and 0 <= col0 and col0 + dim <= table.shape[1], "token_gate: shapes")
+    _check(_lib.mixlib().exl3_mix_token_gate(_p(out), _p(gate_view), _view(gate_view, dim, "gate"), _p(table), table.shape[1], col0, _p(tokens), n, dim, table.shape[0],
+                                              code(out.dtype), _stream(out)))
+
+
+def heads_gate(out: torch.Tensor, a: torch.Tensor, a_row: int, a_head: int, gate_view: torch.Tensor | None, heads: int, vdim: int):
+    """a is addressed as base + n * a_row + h * a_head + v (token-major or head-major); the gate, if any, is [n, heads * vdim] before its sigmoid."""
+    n = out.shape[0]
+    _req(out.is_contiguous() and out.shape == (n, heads * vdim) and a.dtype == out.dtype and a.numel() >= n * heads * vdim, "heads_gate: shapes")
+    if gate_view is not None:
+        _req(gate_view.dtype == out.dtype and gate_view.shape[0] == n, "heads_gate: gate")
+    _check(_lib.mixlib().exl3_mix_heads_gate(_p(out), _p(a), a_row, a_head, _p(gate_view), 0 if gate_view is None else _view(gate_view, heads * vdim, "gate"), n, heads, vdim,
+                                              code(out.dtype), _stream(out)))
+
+
+def topk_sigmoid(idx, wts, logits, correction: torch.Tensor | None, scale: float, normalise: bool = True):
+    n, experts = logits.shape
+    top = idx.shape[1]
+    _f32c(logits, "logits"); _f32c(wts, "wts"); _i32c(idx, "idx")
+    _req(idx.shape == wts.shape == (n, top), "topk_sigmoid: shapes")
+    if correction is not None:
+        _f32c(correction, "correction"); _req(correction.numel() == experts, "topk_sigmoid: correction")
+    _check(_lib.mixlib().exl3_mix_topk_sigmoid(_p(idx), _p(wts), _p(logits), _p(correction), scale, 1 if normalise else 0, n, experts, top, _stream(logits)))
+
+
+# ---- latent attention (csrc/mix_latent.hip) -----------------------------------------------------------------------------------------------------
+def latent_prep(ckr, ring, dkv_view, norm_w, q_view, tok_seq, tok_pos, slots, len_after, freq, mag: float, eps: float, heads: int, dim: int, rot_dim: int, rank: int):
+    n = ckr.shape[0]
+    n_slots, window, row = ring.shape
+    _f32c(norm_w, "norm_w"); _f32c(freq, "freq")
+    _req(row == rank + rot_dim and ckr.shape == (n, row) and ckr.is_contiguous() and ring.is_contiguous() and norm_w.numel() == rank, "latent_prep: cache shapes")
+    _req(ckr.dtype == ring.dtype == dkv_view.dtype == q_view.dtype, "latent_prep: element types")
+    for t, nm in ((tok_seq, "tok_seq"), (tok_pos, "tok_pos"), (slots, "slots"), (len_after, "len_after")):
+        _i32c(t, nm)
+    rot_dims = 2 * freq.numel()
+    _req(tok_seq.numel() == n and tok_pos.numel() == n and dkv_view.shape[0] == n and q_view.shape[0] == n and rot_dims <= rot_dim, "latent_prep: rows")
+    _check(_lib.mixlib().exl3_mix_latent_prep(_p(ckr), _p(ring), _p(dkv_view), _view(dkv_view, row, "dkv"), _p(norm_w), _p(q_view), _view(q_view, heads * (dim + rot_dim), "q"),
+                                               _p(tok_seq), _p(tok_pos), _p(slots), _p(len_after), _p(freq), mag, eps, n, heads, dim, rot_dim, rot_dims, rank, window,
+                                               code(ckr.dtype), _stream(ckr)))
+
+
+def latent_fill_k(k: torch.Tensor, ckr: torch.Tensor, heads: int, dim: int, rot_dim: int, rank: int):
+    n = k.shape[0]
+    _req(k.dtype == ckr.dtype and ckr.is_contiguous() and ckr.shape == (n, rank + rot_dim), "latent_fill_k: shapes")
+    _check(_lib.mixlib().exl3_mix_latent_fill_k(_p(k), _view(k, heads * (dim + rot_dim), "k"), _p(ckr), n, heads, dim, rot_dim, rank, code(k.dtype), _stream(k)))
+
+
+def latent_decode(o_lat: torch.Tensor, q_lat: torch.Tensor, q_view: torch.Tensor, ring: torch.Tensor, sink, slots, len_after, dim: int, rot_dim: int, scale: float):
+    """o_lat, q_lat: [heads, n, rank] (any strides with a unit last one); q_view [n, heads * (dim + rot_dim)] holds the rotated parts."""
+    heads, n, rank = q_lat.shape
+    n_slots, window, row = ring.shape
+    _req(o_lat.shape == q_lat.shape and o_lat.stride(2) == 1 and q_lat.stride(2) == 1 and row == rank + rot_dim and ring.is_contiguous(), "latent_decode: shapes")
+    _req(o_lat.dtype == q_lat.dtype == q_view.dtype == ring.dtype, "latent_decode: element types")
+    _req(slots.numel() == n and len_after.numel() == n and q_view.shape[0] == n, "latent_decode: one row per sequence")
+    if sink is not None:
+        _f32c(sink, "sink"); _req(sink.numel() == heads, "latent_decode: sink")
+    _check(_lib.mixlib().exl3_mix_latent_decode(_p(o_lat), o_lat.stride(1), o_lat.stride(0), _p(q_lat), q_lat.stride(1), q_lat.stride(0), _p(q_view),
+                                                 _view(q_view, heads * (dim + rot_dim), "q"), _p(ring), _p(sink), _p(slots), _p(len_after), n, heads, dim, rot_dim, rank,
+                                                 scale, window, code(o_lat.dtype), _stream(o_lat)))
+
+
+def moe_gate_up_act(hid, h, wg, wu, idx, act_kind: int, limit: float):
+    n, width = h.shape
+    experts, ff, w2 = wg.shape
+    top = idx.shape[1]
+    _req(h.is_contiguous() and wg.is_contiguous() and wu.is_contiguous() and wu.shape == wg.shape and w2 == width and hid.is_contiguous()
+         and hid.shape == (n * top, ff) and hid.dtype == h.dtype == wg.dtype, "moe_gate_up: shapes")
+    _i32c(idx, "idx")
+    _check(_lib.mixlib().exl3_mix_moe_gate_up_act(_p(hid), _p(h), _p(wg), _p(wu), _p(idx), n, top, experts, ff, width, act_kind, limit, code(h.dtype), _stream(h)))

@@ -12,11 +12,21 @@ float32 accumulation; true float32 when the model runs in float32).
     PolyNormMLP             W_down act(W_up h), act = a N(z) + b N(z^2) + c N(z^3) + e
     SparseExperts           top-k of n experts (router in float32, softmax over the chosen logits), experts W_down (silu(W_gate h) * W_up h)
     GatedResidualBlock      x += sublayer(norm(x)) * sigmoid(W norm(x) + b) for a mixer and an optional feed-forward, residual in float32
+    DynTanh                 the norm tanh(alpha x) w + b (no statistics), fused into the residual update that precedes it
+    LatentAttention         attention whose keys and values are up-projections of one cached low-rank latent per token plus one rotated key part
+                            shared by the heads; rotary positions (optionally YaRN-scaled), sliding window, optional sink, optional element-wise
+                            sigmoid output gate; ring cache of [latent | rotated key] per slot; decode in the absorbed form
+    ActMLP                  W_down act(W_up h) with a plain activation (relu^2, gelu, silu)
+    GatedMLP                W_down glu(W_gate h, W_up h) with a gated activation (silu, or the clamped swish with its limit)
+    TokenSide               per-layer token input: a gate on the residual times a slice of a second embedding, projected back and RMS-normed
+    PreNormBlock            x += mixer(norm1(x)); x += ff(norm2(x)); x += side(x), each update fused with what the next consumer reads
+  SparseExperts also routes by sigmoid scores with a selection-only correction, takes either gated activation and an always-on shared expert.
 
 Every sum that the model's exactness rests on (norms, scores, softmax, decays, states, the residual) is float32 inside the kernels in
 both modes; the element type only decides how matrix products and their outputs are held.
 """
 from __future__ import annotations
+from dataclasses import dataclass
 import torch
 import torch.nn.functional as F
 from . import mix_ops
@@ -156,41 +166,278 @@ class PolyNormMLP:
         return F.linear(a, self.w_down), p
 
 
+def rotary_frequencies(dims: int, base: float, scaling: dict | None = None) -> tuple[torch.Tensor, float]:
+    """Per-pair frequencies base^(-2i/dims), i < dims/2, and the magnitude that multiplies cos and sin.  `scaling` (YaRN: factor, original, fast, slow)
+    blends every frequency with its `factor`-times slower version along a linear ramp between the pair indices at which the original context
+    holds `fast` and `slow` turns, and sets the magnitude to 0.1 ln(factor) + 1.  Computed in float64, returned as float32."""
+    import math
+    i = torch.arange(dims // 2, dtype=torch.float64)
+    f = float(base) ** (-2.0 * i / dims)
+    mag = 1.0
+    if scaling is not None:
+        factor, original = float(scaling["factor"]), float(scaling["original"])
+        at = lambda turns: dims * math.log(original / (2.0 * math.pi * turns)) / (2.0 * math.log(float(base)))
+        lo = max(math.floor(at(float(scaling["fast"]))), 0)
+        hi = min(math.ceil(at(float(scaling["slow"]))), dims - 1)
+        ramp = ((i - lo) / max(hi - lo, 0.001)).clamp(0.0, 1.0)
+        f = f / factor * ramp + f * (1.0 - ramp)
+        mag = 0.1 * math.log(factor) + 1.0
+    return f.to(torch.float32), float(mag)
+
+
+class DynTanh:
+    """tanh(alpha x) * w + b: a norm without mean or variance.  It is never a kernel of its own: the residual update before it writes it."""
+
+    def __init__(self, width: int):
+        self.width = width
+
+    def load(self, stc, name: str, device):
+        self.w, self.b = _f32(stc, name, device), _f32(stc, name + ".b", device)
+        self.alpha = float(stc.get_tensor(name + ".alpha", device="cpu").to(torch.float32).reshape(-1)[0])
+        assert self.w.numel() == self.width and self.b.numel() == self.width
+        return self
+
+
+@dataclass
+class NextInput:
+    """What the kernel that updates the residual also writes: the input of the next consumer.  norm None: the stream itself in the activation type."""
+    norm: DynTanh | None
+    out: torch.Tensor            # [n, width] view (any row stride)
+
+
+def update_residual(x: torch.Tensor, y: torch.Tensor | None, nxt: NextInput | None, mode: int = mix_ops.RES_ADD, rms_w: torch.Tensor | None = None, eps: float = 0.0):
+    if nxt is None:
+        if y is not None and mode != mix_ops.RES_KEEP:
+            mix_ops.residual_norm(x, y, mode, rms_w, eps, mix_ops.OUT_NONE, 0.0, None, None, None)
+    elif nxt.norm is None:
+        mix_ops.residual_norm(x, y, mode, rms_w, eps, mix_ops.OUT_CAST, 0.0, None, None, nxt.out)
+    else:
+        mix_ops.residual_norm(x, y, mode, rms_w, eps, mix_ops.OUT_DYN_TANH, nxt.norm.alpha, nxt.norm.w, nxt.norm.b, nxt.out)
+
+
+class LatentAttention:
+    # prompt steps of the same sequence count whose rows all fit the window could skip the ring; nothing of the kind is done: the ring is always written
+    def __init__(self, width: int, heads: int, dim: int, rot_dim: int, vdim: int, rank: int, scale: float, window: int, eps: float, rot_dims: int, rot_base: float,
+                 rot_scaling: dict | None = None, sink: bool = False, gate: bool = False):
+        if rot_dims > rot_dim or rot_dims % 2:
+            raise RuntimeError(f"latent attention: {rot_dims} rotated dimensions of {rot_dim}")
+        if rank > 512:
+            raise RuntimeError("latent attention: the decode kernel holds a latent of at most 512 entries")
+        self.width, self.heads, self.dim, self.rot_dim, self.vdim, self.rank = width, heads, dim, rot_dim, vdim, rank
+        self.scale, self.window, self.eps = float(scale), int(window), float(eps)
+        self.rot_dims, self.rot_base, self.rot_scaling = rot_dims, float(rot_base), rot_scaling
+        self.has_sink, self.has_gate = sink, gate
+        self.qk = dim + rot_dim
+
+    def load(self, stc, prefix: str, dtype, device, extra_parts=()):
+        parts = [("q", _w(stc, prefix + "q", dtype, device), None), ("dkv", _w(stc, prefix + "dkv", dtype, device), None)]
+        if self.has_gate:
+            parts.append(("g", _w(stc, prefix + "g", dtype, device), None))
+        self.inp = FusedInput(parts + list(extra_parts))
+        self.c_norm = _f32(stc, prefix + "dkv.norm", device)
+        w_uk, self.w_uv = _w(stc, prefix + "uk", dtype, device), _w(stc, prefix + "uv", dtype, device)
+        H, d, r, dv, rank = self.heads, self.dim, self.rot_dim, self.vdim, self.rank
+        assert self.inp.offsets["q"][1] == H * self.qk and self.inp.offsets["dkv"][1] == rank + r
+        assert w_uk.shape == (H * d, rank) and self.w_uv.shape == (H * dv, rank)
+        # prompt steps: keys of all heads as ONE product whose result already has room for the rotated part behind every head (zero weight rows there)
+        padded = torch.zeros((H, self.qk, rank), dtype=dtype, device=device)
+        padded[:, :d] = w_uk.view(H, d, rank)
+        self.w_uk_padded = padded.view(H * self.qk, rank)
+        # decode steps, absorbed form: per head q_lat = q_unrotated W_uk[h] and o = o_lat W_uv[h]^T
+        self.w_uk_heads = w_uk.view(H, d, rank)
+        self.w_uv_heads_t = self.w_uv.view(H, dv, rank).transpose(1, 2)
+        self.sink = _f32(stc, prefix + "sink", device) if self.has_sink else None
+        self.w_o = _w(stc, prefix + "o", dtype, device)
+        assert self.w_o.shape == (self.width, H * dv)
+        f, self.rot_mag = rotary_frequencies(self.rot_dims, self.rot_base, self.rot_scaling)
+        self.freq = f.to(device).contiguous()
+        self.dtype = dtype
+
+    def state_specs(self) -> list[StateSpec]:
+        return [StateSpec("ring", (self.window, self.rank + self.rot_dim), self.dtype)]
+
+    def forward(self, h: torch.Tensor, sb: StepBatch, state: dict) -> tuple[torch.Tensor, dict]:
+        H, d, r, dv, rank = self.heads, self.dim, self.rot_dim, self.vdim, self.rank
+        p = self.inp(h)
+        q = p["q"]
+        ckr = torch.empty((sb.n, rank + r), dtype=self.dtype, device=h.device)
+        mix_ops.latent_prep(ckr, state["ring"], p["dkv"], self.c_norm, q, sb.tok_seq, sb.tok_pos, sb.slots, sb.len_after, self.freq, self.rot_mag, self.eps, H, d, r, rank)
+        out = torch.empty((sb.n, H * dv), dtype=self.dtype, device=h.device)
+        if sb.decode:
+            q_heads = q.as_strided((H, sb.n, d), (self.qk, q.stride(0), 1), q.storage_offset())
+            q_lat = torch.bmm(q_heads, self.w_uk_heads)                          # [H, n, rank]
+            o_lat = torch.empty_like(q_lat)
+            mix_ops.latent_decode(o_lat, q_lat, q, state["ring"], self.sink, sb.slots, sb.len_after, d, r, self.scale)
+            o = torch.bmm(o_lat, self.w_uv_heads_t)                              # [H, n, vdim]
+            mix_ops.heads_gate(out, o, dv, sb.n * dv, p.get("g"), H, dv)
+        else:
+            c = ckr[:, :rank]
+            k = F.linear(c, self.w_uk_padded)                                    # [n, H * (d + r)], the rotated slots still zero
+            v = F.linear(c, self.w_uv).view(sb.n, H, dv)
+            mix_ops.latent_fill_k(k, ckr, H, d, r, rank)
+            if self.has_gate:
+                o = torch.empty((sb.n, H * dv), dtype=self.dtype, device=h.device)
+                mix_ops.attn_prefill(o, q, k, v, None, self.sink, sb.cu, sb.tok_seq, sb.tok_pos, H, self.scale, self.window, max_rows=sb.max_rows)
+                mix_ops.heads_gate(out, o, H * dv, dv, p["g"], H, dv)
+            else:
+                mix_ops.attn_prefill(out, q, k, v, None, self.sink, sb.cu, sb.tok_seq, sb.tok_pos, H, self.scale, self.window, max_rows=sb.max_rows)
+        return F.linear(out, self.w_o), p
+
+
+class ActMLP:
+    KINDS = {"relu2": mix_ops.ACT_RELU2, "gelu_tanh": mix_ops.ACT_GELU_TANH, "silu": mix_ops.ACT_SILU}
+
+    def __init__(self, width: int, ff: int, act: str = "relu2"):
+        self.width, self.ff, self.kind = width, ff, self.KINDS[act]
+
+    def load(self, stc, prefix: str, dtype, device, extra_parts=()):
+        self.inp = FusedInput([("up", _w(stc, prefix + "up", dtype, device), None)] + list(extra_parts))
+        self.w_down = _w(stc, prefix + "down", dtype, device)
+        assert self.inp.offsets["up"][1] == self.ff and self.w_down.shape == (self.width, self.ff)
+        self.dtype = dtype
+
+    def forward(self, h: torch.Tensor, sb: StepBatch) -> tuple[torch.Tensor, dict]:
+        p = self.inp(h)
+        a = torch.empty((sb.n, self.ff), dtype=self.dtype, device=h.device)
+        mix_ops.act(a, p["up"], self.kind)
+        return F.linear(a, self.w_down), p
+
+
+class GatedMLP:
+    KINDS = {"silu": mix_ops.GLU_SILU, "clamped_swish": mix_ops.GLU_CLAMPED_SWISH}
+
+    def __init__(self, width: int, ff: int, act: str = "silu", limit: float = 0.0):
+        self.width, self.ff, self.kind, self.limit = width, ff, self.KINDS[act], float(limit)
+
+    def load(self, stc, prefix: str, dtype, device, extra_parts=()):
+        self.inp = FusedInput([("gate", _w(stc, prefix + "gate", dtype, device), None), ("up", _w(stc, prefix + "up", dtype, device), None)] + list(extra_parts))
+        self.w_down = _w(stc, prefix + "down", dtype, device)
+        assert self.inp.offsets["up"][1] == self.ff and self.w_down.shape == (self.width, self.ff)
+        self.dtype = dtype
+
+    def hidden(self, h: torch.Tensor) -> tuple[torch.Tensor, dict]:
+        p = self.inp(h)
+        a = torch.empty((h.shape[0], self.ff), dtype=self.dtype, device=h.device)
+        mix_ops.glu_act(a, p["gate"], p["up"], self.kind, self.limit)
+        return a, p
+
+    def forward(self, h: torch.Tensor, sb: StepBatch, add_to: torch.Tensor | None = None) -> tuple[torch.Tensor, dict]:
+        """add_to: a [n, width] tensor that the down projection is added to (the product's epilogue), e.g. the routed experts' sum."""
+        a, p = self.hidden(h)
+        if add_to is not None:
+            return torch.addmm(add_to, a, self.w_down.t()), p
+        return F.linear(a, self.w_down), p
+
+
+class TokenSide:
+    """x += rms_norm(W_proj (gelu(W_gate x) * e)) * w, e = the layer's slice of a second embedding row of the token.  The gate reads the residual
+    stream itself (in the activation type), not a normed copy."""
+
+    def __init__(self, width: int, dim: int, index: int, eps: float):
+        self.width, self.dim, self.index, self.eps = width, dim, index, float(eps)
+
+    def load(self, stc, prefix: str, table: torch.Tensor, dtype, device):
+        self.table = table                                       # [vocab, layers * dim], shared by the layers
+        self.w_gate, self.w_proj = _w(stc, prefix + "gate", dtype, device), _w(stc, prefix + "proj", dtype, device)
+        self.norm_w = _f32(stc, prefix + "norm", device)
+        assert self.w_gate.shape == (self.dim, self.width) and self.w_proj.shape == (self.width, self.dim) and (self.index + 1) * self.dim <= table.shape[1]
+        self.dtype = dtype
+
+    def forward(self, xc: torch.Tensor, sb: StepBatch) -> torch.Tensor:
+        gate = F.linear(xc, self.w_gate)
+        g = torch.empty((sb.n, self.dim), dtype=self.dtype, device=xc.device)
+        mix_ops.token_gate(g, gate, self.table, self.index * self.dim, sb.tokens)
+        return F.linear(g, self.w_proj)
+
+
+class PreNormBlock:
+    """x += mixer(norm1(x)); x += ff(norm2(x)) (if a feed-forward); x += side(x) (if a token side input).  Every update of the float32 residual is one
+    kernel that also writes what comes next: the next norm's output, or the stream in the activation type."""
+
+    def __init__(self, width: int, eps: float, mixer, mlp, side: TokenSide | None):
+        self.width, self.eps, self.mixer, self.mlp, self.side = width, float(eps), mixer, mlp, side
+        self.norm1, self.norm2 = DynTanh(width), (DynTanh(width) if mlp is not None else None)
+
+    def load(self, stc, prefix: str, dtype, device, side_table: torch.Tensor | None = None):
+        self.norm1.load(stc, prefix + "norm1", device)
+        self.mixer.load(stc, prefix + "mix.", dtype, device)
+        if self.mlp is not None:
+            self.norm2.load(stc, prefix + "norm2", device)
+            self.mlp.load(stc, prefix + "mlp.", dtype, device)
+        if self.side is not None:
+            self.side.load(stc, prefix + "side.", side_table, dtype, device)
+        self.dtype = dtype
+
+    def state_specs(self) -> list[StateSpec]:
+        return self.mixer.state_specs()
+
+    def forward(self, x: torch.Tensor, h: torch.Tensor, sb: StepBatch, state: dict, nxt: NextInput | None):
+        """x: float32 residual (updated in place); h = norm1(x).  nxt: what the block's last update writes for whoever reads the stream next."""
+        new = lambda: torch.empty((sb.n, self.width), dtype=self.dtype, device=x.device)
+        y, _ = self.mixer.forward(h, sb, state)
+        if self.mlp is not None:
+            h2 = new()
+            update_residual(x, y, NextInput(self.norm2, h2))
+            y, _ = self.mlp.forward(h2, sb)
+        if self.side is None:
+            update_residual(x, y, nxt)
+            return
+        xc = new()
+        update_residual(x, y, NextInput(None, xc))
+        update_residual(x, self.side.forward(xc, sb), nxt, rms_w=self.side.norm_w, eps=self.eps)
+
+
 class SparseExperts:
     # rows from which the expert-sorted matrix products take over from the weight-streaming kernels, and rows from which the streaming kernels
     # walk each chosen expert once for all its rows instead of once per (row, choice)
     GROUPED_MIN_ROWS = 64
     EXPERT_MAJOR_MIN_ROWS = 4
 
-    def __init__(self, width: int, ff: int, experts: int, top: int):
+    def __init__(self, width: int, ff: int, experts: int, top: int, router: str = "softmax", router_bias: bool = True, correction: bool = False,
+                 route_scale: float = 1.0, act: str = "silu", limit: float = 0.0, shared: GatedMLP | None = None):
+        """router "softmax": the top logits, weights = softmax over them.  "sigmoid": scores sigmoid(z), chosen by score (+ a stored correction that the
+        weights do not see), weights = chosen scores / their sum * route_scale.  shared: an expert that every row runs, added to the routed sum."""
         if not 0 < top <= experts:
             raise RuntimeError(f"router: top {top} of {experts} experts")
+        if router not in ("softmax", "sigmoid"):
+            raise RuntimeError(f"router: unknown kind {router!r}")
         self.width, self.ff, self.experts, self.top = width, ff, experts, top
+        self.router, self.has_router_bias, self.has_correction, self.route_scale = router, router_bias, correction, float(route_scale)
+        self.act_kind, self.limit, self.shared = GatedMLP.KINDS[act], float(limit), shared
 
     def load(self, stc, prefix: str, dtype, device, extra_parts=()):
         stack = lambda nm: torch.stack([_w(stc, f"{prefix}e{e}.{nm}", dtype, device) for e in range(self.experts)]).contiguous()
         self.w_gate, self.w_up, self.w_down = stack("gate"), stack("up"), stack("down")
         self.w_router = _f32(stc, prefix + "router", device)
-        self.b_router = _f32(stc, prefix + "router.b", device)
+        self.b_router = _f32(stc, prefix + "router.b", device) if self.has_router_bias else None
+        self.correction = _f32(stc, prefix + "correction", device) if self.has_correction else None
+        if self.shared is not None:
+            self.shared.load(stc, prefix + "shared.", dtype, device)
         self.inp = FusedInput(list(extra_parts)) if extra_parts else None
         assert self.w_gate.shape == (self.experts, self.ff, self.width) and self.w_down.shape == (self.experts, self.width, self.ff)
         self.dtype = dtype
 
     def forward(self, h: torch.Tensor, sb: StepBatch) -> tuple[torch.Tensor, dict]:
         p = self.inp(h) if self.inp is not None else {}
-        logits = torch.addmm(self.b_router, h.float(), self.w_router.t())          # float32 product of the (rounded) input
+        hf = h.float()                                                              # float32 product of the (rounded) input
+        logits = torch.addmm(self.b_router, hf, self.w_router.t()) if self.b_router is not None else torch.mm(hf, self.w_router.t())
         idx = torch.empty((sb.n, self.top), dtype=torch.int32, device=h.device)
         wts = torch.empty((sb.n, self.top), dtype=torch.float32, device=h.device)
-        mix_ops.topk_softmax(idx, wts, logits)
+        if self.router == "softmax":
+            mix_ops.topk_softmax(idx, wts, logits)
+        else:
+            mix_ops.topk_sigmoid(idx, wts, logits, self.correction, self.route_scale)
         y = torch.empty((sb.n, self.width), dtype=self.dtype, device=h.device)
         if sb.n >= self.GROUPED_MIN_ROWS:
-            mix_ops.moe_grouped(y, h, self.w_gate, self.w_up, self.w_down, idx, wts)
+            mix_ops.moe_grouped(y, h, self.w_gate, self.w_up, self.w_down, idx, wts, self.act_kind, self.limit)
         elif sb.n >= self.EXPERT_MAJOR_MIN_ROWS and mix_ops.moe_vector_layout(h, self.ff):
-            mix_ops.moe_expert_major(y, h, self.w_gate, self.w_up, self.w_down, idx, wts)
+            mix_ops.moe_expert_major(y, h, self.w_gate, self.w_up, self.w_down, idx, wts, self.act_kind, self.limit)
         else:
             hid = torch.empty((sb.n * self.top, self.ff), dtype=self.dtype, device=h.device)
-            mix_ops.moe_gate_up(hid, h, self.w_gate, self.w_up, idx)
+            mix_ops.moe_gate_up_act(hid, h, self.w_gate, self.w_up, idx, self.act_kind, self.limit)
             mix_ops.moe_down(y, hid, self.w_down, idx, wts)
+        if self.shared is not None:
+            y, _ = self.shared.forward(h, sb, add_to=y)
         return y, p
 
 

@@ -3,7 +3,7 @@ Model registry: config.json names an architecture, the registry maps it to the c
 
     load_model(directory, device, dtype)  ->  a model with  .vocab, .new_cache(slots), .step(StepBatch, cache) -> float32 logits
 
-Registered: the unquantized mixer family (Vofanex) with the step interface above, and the EXL3-quantized Llama of llama_path.py, which
+Registered: the unquantized mixer families (Vofanex, Zagilorn) with the step interface above, and the EXL3-quantized Llama of llama_path.py, which
 keeps its own decode_step / prefill_chunk pipelines (`load_model` returns it for `LlamaForCausalLM` checkpoints; the token-level
 generator drives step-interface models only).
 """
@@ -13,13 +13,21 @@ import os
 import torch
 
 _REGISTRY: dict[str, callable] = {}
+_LIBRARIES: dict[str, tuple] = {}
 
 
-def register(architecture: str):
+def register(architecture: str, libraries: tuple = ("hip",)):
+    """libraries: the native libraries the architecture's kernels live in ("mix": libexl3_mix.so, "hip": libexl3_hip.so) -- what a fresh checkout compiles
+    before the model is loaded."""
     def deco(fn):
         _REGISTRY[architecture] = fn
+        _LIBRARIES[architecture] = tuple(libraries)
         return fn
     return deco
+
+
+def native_libraries(architecture: str) -> tuple:
+    return _LIBRARIES.get(architecture, ("hip",))
 
 
 def architectures() -> list[str]:
@@ -45,10 +53,16 @@ def load_model(directory: str, device="cuda:0", dtype: torch.dtype | None = None
     return _REGISTRY[a](directory, config, device, dtype)
 
 
-@register("Vofanex")
+@register("Vofanex", libraries=("mix",))
 def _load_vofanex(directory, config, device, dtype):
     from .vofanex import VofanexModel
     return VofanexModel.from_directory(directory, device=device, dtype=dtype or torch.bfloat16)
+
+
+@register("Zagilorn", libraries=("mix",))
+def _load_zagilorn(directory, config, device, dtype):
+    from .zagilorn import ZagilornModel
+    return ZagilornModel.from_directory(directory, device=device, dtype=dtype or torch.bfloat16)
 
 
 @register("LlamaForCausalLM")

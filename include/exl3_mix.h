@@ -2,7 +2,8 @@
  * exl3_mix.h -- C-ABI of the sequence-mixer library (libexl3_mix.so): the kernels of models whose layers are not the
  * quantized-linear transformer block of libexl3_hip.so -- sliding-window attention with a learned sink over a ring cache, gated
  * linear attention with a per-channel decay and a carried state, RMS norms over a 32-bit residual stream, a gated residual,
- * the PolyNorm activation, a top-k router and unquantized experts.
+ * the PolyNorm activation, top-k routers and unquantized experts; latent attention (a low-rank key/value cache with rotary positions), the
+ * Dynamic Tanh norm and the residual updates of pre-norm blocks.
  *
  * Conventions (the same as exl3_hip.h): plain device pointers, sizes and scalars; `stream` is a hipStream_t; calls are
  * asynchronous; return 0 on success and < 0 on error with the text in exl3_mix_last_error() (thread-local).
@@ -32,7 +33,16 @@ extern "C" {
 #define EXL3_MIX_BF16 0
 #define EXL3_MIX_F32  1
 
-#define EXL3_MIX_ABI_VERSION 1
+/* gated activations of two projections g (gate) and u (up):  SILU: silu(g) u;  CLAMPED_SWISH: g' = min(g, limit), u' = clamp(u, -limit, limit),
+ * g' sigmoid(1.702 g') (u' + 1). */
+#define EXL3_MIX_GLU_SILU          0
+#define EXL3_MIX_GLU_CLAMPED_SWISH 1
+/* plain activations */
+#define EXL3_MIX_ACT_RELU2     0
+#define EXL3_MIX_ACT_GELU_TANH 1
+#define EXL3_MIX_ACT_SILU      2
+
+#define EXL3_MIX_ABI_VERSION 2
 
 const char* exl3_mix_last_error(void);
 int  exl3_mix_abi_version(void);
@@ -122,6 +132,62 @@ int exl3_mix_moe_expert_major(void* per, void* hid, const void* h, const void* w
  * out = silu(g) * u element by element, and y[n] = sum_r wts[n][r] * sorted[where[n*top + r]] (rows back in token order, weighted). */
 int exl3_mix_silu_mul(void* out, const void* g, const void* u, int64_t count, int dtype, void* stream);
 int exl3_mix_moe_combine(void* y, const void* sorted, const int32_t* where, const float* wts, int n, int top, int width, int dtype, void* stream);
+
+/* The same experts with the gated activation named by `act` (EXL3_MIX_GLU_*) and its clamp `limit`. */
+int exl3_mix_moe_gate_up_act(void* hid, const void* h, const void* wg, const void* wu, const int32_t* idx, int n, int top, int experts, int ff, int width,
+                             int act, float limit, int dtype, void* stream);
+int exl3_mix_moe_expert_major_act(void* per, void* hid, const void* h, const void* wg, const void* wu, const void* wd, const int32_t* idx,
+                                  int n, int top, int experts, int ff, int width, int act, float limit, int dtype, void* stream);
+
+/* ---- pre-norm blocks whose norm needs no statistics, and the pieces between their matrix products (mix_rowops.hip) ---- */
+
+/* x[n] = table[tokens[n]] (float32 residual); if xc: the same row in the activation type at xc + n * xc_ld. */
+int exl3_mix_embed_copy(float* x, void* xc, int64_t xc_ld, const void* table, const int32_t* tokens, int n, int width, int vocab, int dtype, void* stream);
+
+/* Residual update fused with what the next consumer reads.  mode 0: x stays (y unused); 1: x += y'; 2: x = y', where y' = y, or, with rms_w,
+ * y / sqrt(mean(y^2) + eps) * rms_w.  out 0: nothing; 1: h = x in the activation type; 2: h = tanh(alpha x) * w + b (Dynamic Tanh: no mean, no
+ * variance).  y and h may be column blocks (row strides y_ld, h_ld). */
+int exl3_mix_residual_norm(float* x, const void* y, int64_t y_ld, int mode, const float* rms_w, float eps, int out, float alpha, const float* w, const float* b,
+                           void* h, int64_t h_ld, int n, int width, int dtype, void* stream);
+
+/* h[i] = tanh(alpha * x[rows ? rows[i] : i]) * w + b: the last norm on the wanted rows only. */
+int exl3_mix_dyn_tanh_rows(void* h, const float* x, const int32_t* rows, float alpha, const float* w, const float* b, int n, int width, int dtype, void* stream);
+
+/* out[n][i] = act(z[n][i]) (EXL3_MIX_ACT_*), and out[n][i] = glu(g[n][i], u[n][i]) (EXL3_MIX_GLU_*, `limit` for the clamped kind); out is contiguous. */
+int exl3_mix_act(void* out, const void* z, int64_t z_ld, int n, int ff, int kind, int dtype, void* stream);
+int exl3_mix_glu_act(void* out, const void* g, int64_t g_ld, const void* u, int64_t u_ld, int n, int ff, int kind, float limit, int dtype, void* stream);
+
+/* out[n][j] = gelu_tanh(gate[n][j]) * table[tokens[n]][col0 + j], j < dim: a gate multiplied with a slice of a per-token embedding row. */
+int exl3_mix_token_gate(void* out, const void* gate, int64_t gate_ld, const void* table, int64_t table_ld, int col0, const int32_t* tokens,
+                        int n, int dim, int vocab, int dtype, void* stream);
+
+/* out[n][h * vdim + v] = a[n * a_row + h * a_head + v] * (gate ? sigmoid(gate[n][h * vdim + v]) : 1): an element-wise output gate over heads that may lie
+ * head-major (the result of a per-head batched product). */
+int exl3_mix_heads_gate(void* out, const void* a, int64_t a_row, int64_t a_head, const void* gate, int64_t gate_ld, int n, int heads, int vdim, int dtype, void* stream);
+
+/* Router with independent scores s = sigmoid(z): the `top` experts with the largest s + correction (correction may be NULL; ties go to the lower index);
+ * weights = s / (sum of the chosen s + 1e-20) * scale, or s * scale with normalise = 0. */
+int exl3_mix_topk_sigmoid(int32_t* idx, float* wts, const float* logits, const float* correction, float scale, int normalise, int n, int experts, int top, void* stream);
+
+/* ---- latent attention (mix_latent.hip): per token one low-rank latent c [rank] and one rotated key part k_rot [rot_dim] shared by all heads ---- */
+
+/* From dkv [n][rank + rot_dim]: c = rms_norm(dkv[:rank]) * norm_w; k_rot = the rest with rotary positions on its first rot_dims entries (interleaved
+ * pairs (2i, 2i+1), angle = tok_pos * freq[i], cos and sin times `mag`, all float32).  [c | k_rot] goes to ckr [n][rank + rot_dim] and, for the rows among
+ * the last `window` positions of their sequence, to ring [slots][window][rank + rot_dim] at tok_pos % window.  The same rotation is applied in place to
+ * the last rot_dim entries of every head of q [n][heads][dim + rot_dim]. */
+int exl3_mix_latent_prep(void* ckr, void* ring, const void* dkv, int64_t dkv_ld, const float* norm_w, void* q, int64_t q_ld,
+                         const int32_t* tok_seq, const int32_t* tok_pos, const int32_t* slots, const int32_t* len_after,
+                         const float* freq, float mag, float eps, int n, int heads, int dim, int rot_dim, int rot_dims, int rank, int window, int dtype, void* stream);
+
+/* k [n][heads][dim + rot_dim]: the last rot_dim entries of every head = k_rot of the row (ckr as written by exl3_mix_latent_prep). */
+int exl3_mix_latent_fill_k(void* k, int64_t k_ld, const void* ckr, int n, int heads, int dim, int rot_dim, int rank, int dtype, void* stream);
+
+/* One new row per sequence against the ring in the absorbed form: score_j = scale * (q_lat . c_j + q_rot . k_rot_j) over the min(len_after, window) newest
+ * entries, softmax (with exp(sink_h) in the denominator if sink), o_lat = sum_j w_j c_j.  q_lat (the head's unrotated query carried into the latent space)
+ * and o_lat are addressed as base + n * row_stride + h * head_stride; q_rot is read from q [n][heads][dim + rot_dim].  rank <= 512. */
+int exl3_mix_latent_decode(void* o_lat, int64_t o_row, int64_t o_head, const void* q_lat, int64_t ql_row, int64_t ql_head, const void* q, int64_t q_ld,
+                           const void* ring, const float* sink, const int32_t* slots, const int32_t* len_after,
+                           int n, int heads, int dim, int rot_dim, int rank, float scale, int window, int dtype, void* stream);
 
 #ifdef __cplusplus
 }
