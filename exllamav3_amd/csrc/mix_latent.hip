@@ -126,17 +126,17 @@ extern "C" int exl3_mix_latent_decode(void* o_lat, int64_t o_row, int64_t o_head
                                       int n, int heads, int dim, int rot_dim, int rank, float scale, int window, int dtype, void* stream)
 {
     MIX_CHECK(o_lat && q_lat && q && ring && slots && len_after, "mix_latent_decode: null pointer");
-    MIX_CHECK(n >= 0 && heads > 0 && heads <= 65535 && dim >= 0 && rot_dim >= 0 && rank > 0 && rank <= 512 && rank + rot_dim <= 4096 && window > 0,
-              "mix_latent_decode: rank %d (<= 512) / rot_dim %d / window %d out of range", rank, rot_dim, window);
+    MIX_CHECK(n >= 0 && heads > 0 && heads <= 65535 && dim >= 0 && rot_dim >= 0 && rank > 0 && rank <= 1024 && rank + rot_dim <= 4096 && window > 0,
+              "mix_latent_decode: rank %d (<= 1024) / rot_dim %d / window %d out of range", rank, rot_dim, window);
     MIX_CHECK(q_ld >= (int64_t) heads * (dim + rot_dim), "mix_latent_decode: bad row stride");
     if (n == 0) return EXL3_MIX_OK;
     const int mv = (rank + 63) / 64;
-    const int mvt = mv == 1 ? 1 : (mv == 2 ? 2 : (mv <= 4 ? 4 : 8));
+    const int mvt = mv == 1 ? 1 : (mv == 2 ? 2 : (mv <= 4 ? 4 : (mv <= 8 ? 8 : 16)));
     const size_t sm = (size_t) (rank + rot_dim + AT_WAVES * 64 + AT_WAVES * (2 + mvt * 64)) * sizeof(float);
     #define LD_LAUNCH(MV) hipLaunchKernelGGL((latent_decode_kernel<T, MV>), dim3(n, heads), dim3(64 * AT_WAVES), sm, (hipStream_t) stream, (T*) o_lat, o_row, o_head, \
                                              (const T*) q_lat, ql_row, ql_head, (const T*) q, q_ld, (const T*) ring, sink, slots, len_after, dim, rot_dim, rank, scale, window)
     MIX_DISPATCH_T(dtype,
-        if (mv == 1) LD_LAUNCH(1); else if (mv == 2) LD_LAUNCH(2); else if (mv <= 4) LD_LAUNCH(4); else LD_LAUNCH(8));
+        if (mv == 1) LD_LAUNCH(1); else if (mv == 2) LD_LAUNCH(2); else if (mv <= 4) LD_LAUNCH(4); else if (mv <= 8) LD_LAUNCH(8); else LD_LAUNCH(16));
     #undef LD_LAUNCH
     return mix_check_launch("mix_latent_decode");
 }

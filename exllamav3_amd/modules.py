@@ -216,13 +216,12 @@ def update_residual(x: torch.Tensor, y: torch.Tensor | None, nxt: NextInput | No
 
 
 class LatentAttention:
-    # prompt steps of the same sequence count whose rows all fit the window could skip the ring; nothing of the kind is done: the ring is always written
     def __init__(self, width: int, heads: int, dim: int, rot_dim: int, vdim: int, rank: int, scale: float, window: int, eps: float, rot_dims: int, rot_base: float,
                  rot_scaling: dict | None = None, sink: bool = False, gate: bool = False):
         if rot_dims > rot_dim or rot_dims % 2:
             raise RuntimeError(f"latent attention: {rot_dims} rotated dimensions of {rot_dim}")
-        if rank > 512:
-            raise RuntimeError("latent attention: the decode kernel holds a latent of at most 512 entries")
+        if rank > 1024:
+            raise RuntimeError("latent attention: the decode kernel holds a latent of at most 1024 entries")
         self.width, self.heads, self.dim, self.rot_dim, self.vdim, self.rank = width, heads, dim, rot_dim, vdim, rank
         self.scale, self.window, self.eps = float(scale), int(window), float(eps)
         self.rot_dims, self.rot_base, self.rot_scaling = rot_dims, float(rot_base), rot_scaling

@@ -184,7 +184,7 @@ int exl3_mix_latent_fill_k(void* k, int64_t k_ld, const void* ckr, int n, int he
 
 /* One new row per sequence against the ring in the absorbed form: score_j = scale * (q_lat . c_j + q_rot . k_rot_j) over the min(len_after, window) newest
  * entries, softmax (with exp(sink_h) in the denominator if sink), o_lat = sum_j w_j c_j.  q_lat (the head's unrotated query carried into the latent space)
- * and o_lat are addressed as base + n * row_stride + h * head_stride; q_rot is read from q [n][heads][dim + rot_dim].  rank <= 512. */
+ * and o_lat are addressed as base + n * row_stride + h * head_stride; q_rot is read from q [n][heads][dim + rot_dim].  rank <= 1024. */
 int exl3_mix_latent_decode(void* o_lat, int64_t o_row, int64_t o_head, const void* q_lat, int64_t ql_row, int64_t ql_head, const void* q, int64_t q_ld,
                            const void* ring, const float* sink, const int32_t* slots, const int32_t* len_after,
                            int n, int heads, int dim, int rot_dim, int rank, float scale, int window, int dtype, void* stream);
