@@ -55,6 +55,8 @@ def parse():
     ap.add_argument("--prefill-tokens", type=int, default=4096)
     ap.add_argument("--mixer-family", action="store_true",
                     help="instead of the default workload: layer times of the unquantized mixer family (Vofanex) beside the EXL3 Llama layer of equal size, and its kernels' rooflines")
+    ap.add_argument("--latent-family", action="store_true",
+                    help="instead of the default workload: layer times of the latent-attention family (Zagilorn) beside Vofanex layers of equal size, and its kernels' rooflines")
     ap.add_argument("--mixer-sizes", default="", help="with --mixer-family: comma-separated sizes (1b, 8b; default both)")
     ap.add_argument("--variant", type=int, default=1)
     ap.add_argument("--attention", action="store_true", help="include decode attention over the quantized KV cache (context = 1000 tokens) in the timed step")
@@ -254,6 +256,9 @@ def main():
     if args.mixer_family:
         from exllamav3_amd import mixer_bench
         sys.exit(mixer_bench.run(args))
+    if args.latent_family:
+        from exllamav3_amd import latent_bench
+        sys.exit(latent_bench.run(args))
     import torch
     from exllamav3_amd import ext
     from exllamav3_amd.llama_path import SHAPES, SyntheticEXL3Llama

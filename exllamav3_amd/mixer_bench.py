@@ -85,15 +85,19 @@ def _time(fn, n, warm=2):
     return e0.elapsed_time(e1) / n * 1e-3
 
 
-def model_legs(size_name: str, prompt: int, ctx: int, steps: int, dev):
-    """Per layer kind: prefill seconds per layer at `prompt` rows, decode seconds per layer at batch 1 and 16 after `ctx` tokens (eager, and batch 1 as a captured graph)."""
+def _make_vofanex(size, kind, reps, dev):
     from .vofanex import VofanexModel
+    cfg, td = synth(size, [kind] * reps, device=dev)
+    return VofanexModel(cfg, td, device=dev, dtype=torch.bfloat16)
+
+
+def model_legs(size_name: str, prompt: int, ctx: int, steps: int, dev, kinds=None, make=_make_vofanex):
+    """Per layer kind: prefill seconds per layer at `prompt` rows, decode seconds per layer at batch 1 and 16 after `ctx` tokens (eager, and batch 1 as a captured graph).
+    make(size, kind, reps, dev) builds a step-interface model of `reps` layers of one kind."""
     size, out = SIZES[size_name], {}
-    for kind in LAYER_KINDS:
+    for kind in (kinds or LAYER_KINDS):
         reps = 2
-        cfg, td = synth(size, [kind] * reps, device=dev)
-        m = VofanexModel(cfg, td, device=dev, dtype=torch.bfloat16)
-        del td
+        m = make(size, kind, reps, dev)
         cache = m.new_cache(16)
         toks = torch.randint(0, 32000, (prompt,)).tolist()
         slots = [cache.alloc() for _ in range(16)]
