@@ -323,4 +323,6 @@ def _declare_mix(l):
     sig("exl3_mix_topk_sigmoid", vp, vp, vp, vp, f32, i32, i32, i32, i32, vp)
     sig("exl3_mix_latent_prep", vp, vp, vp, i64, vp, vp, i64, vp, vp, vp, vp, vp, f32, f32, i32, i32, i32, i32, i32, i32, i32, i32, vp)
     sig("exl3_mix_latent_fill_k", vp, i64, vp, i32, i32, i32, i32, i32, i32, vp)
+    sig("exl3_mix_latent_decode_mfma_scratch", i32, i32, i32, i32, ctypes.POINTER(i64))
+    sig("exl3_mix_latent_decode_mfma", vp, i64, i64, vp, i64, i64, vp, i64, vp, vp, vp, vp, vp, i32, i32, i32, i32, i32, i32, f32, i32, vp)
     sig("exl3_mix_latent_decode", vp, i64, i64, vp, i64, i64, vp, i64, vp, vp, vp, vp, i32, i32, i32, i32, i32, f32, i32, i32, vp)

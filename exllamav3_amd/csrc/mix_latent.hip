@@ -8,6 +8,9 @@
 //   latent_decode   decode steps in the ABSORBED form: the query is carried into the latent space (q_lat = W_uk^T q per head, a vendor product), the
 //                   cached [c | k_rot] rows are the keys of every head and c is also the value; the result is a weighted latent per head that the
 //                   caller up-projects with W_uv.  Scores, softmax and sums are the float32 row worker of mix_attn_row.cuh.
+//   latent_decode_mfma   the same on the matrix cores (bfloat16): all heads of a sequence score the SAME cached rows, so sixteen heads are the
+//                   sixteen columns of one MFMA tile and every cached row is read once per sixteen heads instead of once per head.  The keys of a
+//                   sequence are split over workgroups of one wave; a second kernel merges the partial sums (and adds the sink).
 #include "mix_common.cuh"
 #include "mix_attn_row.cuh"
 
@@ -20,6 +23,7 @@ __global__ __launch_bounds__(256) void latent_prep_kernel(T* __restrict__ ckr, T
                                                           int heads, int dim, int rot_dim, int rot_dims, int rank, int window)
 {
     __shared__ float red[4];
+    extern __shared__ float trig[];                            // [pairs][2]: cos, sin of the row's position, computed once for the key part and every head
     const int n = blockIdx.x;
     const int b = tok_seq[n], pos = tok_pos[n];
     const bool keep = pos >= len_after[b] - window;
@@ -39,11 +43,17 @@ __global__ __launch_bounds__(256) void latent_prep_kernel(T* __restrict__ ckr, T
     }
     const int pairs = rot_dims / 2;
     const float p = (float) pos;
+    for (int i = threadIdx.x; i < pairs; i += 256)
+    {
+        float sn, cs;
+        sincosf(p * freq[i], &sn, &cs);
+        trig[2 * i] = cs * mag; trig[2 * i + 1] = sn * mag;
+    }
+    __syncthreads();
     // the shared key part: rotated pairs, then what lies beyond rot_dims unchanged
     for (int i = threadIdx.x; i < pairs; i += 256)
     {
-        const float a = p * freq[i];
-        const float cs = cosf(a) * mag, sn = sinf(a) * mag;
+        const float cs = trig[2 * i], sn = trig[2 * i + 1];
         const float u = to_f(src[rank + 2 * i]), v = to_f(src[rank + 2 * i + 1]);
         const T o0 = from_f<T>(u * cs - v * sn), o1 = from_f<T>(v * cs + u * sn);
         dst[rank + 2 * i] = o0; dst[rank + 2 * i + 1] = o1;
@@ -60,8 +70,7 @@ __global__ __launch_bounds__(256) void latent_prep_kernel(T* __restrict__ ckr, T
     for (int t = threadIdx.x; t < heads * pairs; t += 256)
     {
         const int h = t / pairs, i = t - h * pairs;
-        const float a = p * freq[i];
-        const float cs = cosf(a) * mag, sn = sinf(a) * mag;
+        const float cs = trig[2 * i], sn = trig[2 * i + 1];
         T* e = qr + (int64_t) h * (dim + rot_dim) + dim + 2 * i;
         const float u = to_f(e[0]), v = to_f(e[1]);
         e[0] = from_f<T>(u * cs - v * sn);
@@ -108,7 +117,7 @@ extern "C" int exl3_mix_latent_prep(void* ckr, void* ring, const void* dkv, int6
     MIX_CHECK(rot_dims >= 0 && rot_dims <= rot_dim && rot_dims % 2 == 0, "mix_latent_prep: %d rotated dimensions of %d", rot_dims, rot_dim);
     MIX_CHECK(dkv_ld >= rank + rot_dim && q_ld >= (int64_t) heads * (dim + rot_dim), "mix_latent_prep: bad row strides");
     if (n == 0) return EXL3_MIX_OK;
-    MIX_DISPATCH_T(dtype, hipLaunchKernelGGL(latent_prep_kernel<T>, dim3(n), dim3(256), 0, (hipStream_t) stream, (T*) ckr, (T*) ring, (const T*) dkv, dkv_ld, norm_w,
+    MIX_DISPATCH_T(dtype, hipLaunchKernelGGL(latent_prep_kernel<T>, dim3(n), dim3(256), (size_t) (rot_dims + 2) * sizeof(float), (hipStream_t) stream, (T*) ckr, (T*) ring, (const T*) dkv, dkv_ld, norm_w,
                                              (T*) q, q_ld, tok_seq, tok_pos, slots, len_after, freq, mag, eps, heads, dim, rot_dim, rot_dims, rank, window));
     return mix_check_launch("mix_latent_prep");
 }
@@ -139,4 +148,188 @@ extern "C" int exl3_mix_latent_decode(void* o_lat, int64_t o_row, int64_t o_head
         if (mv == 1) LD_LAUNCH(1); else if (mv == 2) LD_LAUNCH(2); else if (mv <= 4) LD_LAUNCH(4); else if (mv <= 8) LD_LAUNCH(8); else LD_LAUNCH(16));
     #undef LD_LAUNCH
     return mix_check_launch("mix_latent_decode");
+}
+
+// ---- decode on the matrix cores ---------------------------------------------------------------------------------------------------------------
+// One wave = one split of one sequence's cached rows x one group of 16 heads.  v_mfma_f32_16x16x32_bf16 operand lane (g = lane / 16, c = lane % 16)
+// holds row / column c and contraction slots 8g .. 8g+7; result lane (g, c) holds rows 4g .. 4g+3 of column c.
+//   scores, transposed: S^T = K Q^T.  A = 16 cached rows (lane: row c, 16 bytes straight from the ring, no staging), B = the 16 heads' absorbed queries
+//   [q_lat | q_rot] (registers, loaded once).  A lane then holds the scores of ONE head, so the running maximum and sum are per-lane scalars.
+//   O^T = C^T P^T over tiles of 32 keys: the score registers of two 16-key tiles are the B operand as they stand when contraction slot (g, e) means key
+//   4g + e of the first tile (e < 4) or of the second (e >= 4); A = the latent columns of the same rows, transposed through LDS (the rows are in registers
+//   already: they were the A operands of the scores).
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+#define LM_KEYS 32
+#define LM_VS (LM_KEYS + 8)
+
+template <int NV, int KD>
+__global__ __launch_bounds__(64) void latent_decode_mfma_kernel(float* __restrict__ part_o, float* __restrict__ part_ml, const bf16_t* __restrict__ q_lat, int64_t ql_row,
+                                                                 int64_t ql_head, const bf16_t* __restrict__ q, int64_t q_ld, const bf16_t* __restrict__ ring,
+                                                                 const int32_t* __restrict__ slots, const int32_t* __restrict__ len_after,
+                                                                 int heads, int dim, int rot_dim, int rank, float scale, int window, int keys_per_split)
+{
+    __shared__ __attribute__((aligned(16))) uint16_t vt[NV * 16 * LM_VS];        // [latent column][key of the tile]
+    const int sp = blockIdx.x, hg = blockIdx.y, n = blockIdx.z, splits = gridDim.x;
+    const int lane = threadIdx.x, g = lane >> 4, c = lane & 15;
+    const int count = min(len_after[n], window);
+    const int k_begin = sp * keys_per_split, k_end = min(count, k_begin + keys_per_split);
+    const int row = rank + rot_dim;
+    const bf16_t* kb = ring + (int64_t) slots[n] * window * row;
+    const int head = hg * 16 + c;
+    const bool head_ok = head < heads;
+    const int64_t pidx = ((int64_t) n * splits + sp) * heads + head;
+    if (k_begin >= k_end)
+    {
+        if (head_ok && g == 0) { part_ml[pidx * 2] = -INFINITY; part_ml[pidx * 2 + 1] = 0.f; }
+        return;
+    }
+    bf16x8 qf[KD];
+    #pragma unroll
+    for (int s = 0; s < KD; ++s)
+    {
+        union { bf16x8 v; uint16_t u[8]; } t;
+        #pragma unroll
+        for (int e = 0; e < 8; ++e)
+        {
+            const int col = s * 32 + g * 8 + e;
+            uint16_t x = 0;
+            if (head_ok && col < rank) x = q_lat[(int64_t) n * ql_row + (int64_t) head * ql_head + col].u;
+            else if (head_ok && col < row) x = q[(int64_t) n * q_ld + (int64_t) head * (dim + rot_dim) + dim + (col - rank)].u;
+            t.u[e] = x;
+        }
+        qf[s] = t.v;
+    }
+    float m = -1e30f, l = 0.f;
+    f32x4 acc[NV];
+    #pragma unroll
+    for (int t = 0; t < NV; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int j0 = k_begin; j0 < k_end; j0 += LM_KEYS)
+    {
+        __syncthreads();                                           // one wave: the previous tile's operand reads are over
+        f32x4 sc[2] = {f32x4{0.f, 0.f, 0.f, 0.f}, f32x4{0.f, 0.f, 0.f, 0.f}};
+        #pragma unroll
+        for (int s = 0; s < KD; ++s)
+        {
+            #pragma unroll
+            for (int u = 0; u < 2; ++u)
+            {
+                const int jr = min(j0 + u * 16 + c, count - 1);   // rows past the split are read (they exist) and masked below
+                const int col0 = s * 32 + g * 8;                  // row is a multiple of 8: a group of 8 columns is inside the row or outside
+                union { bf16x8 v; uint4 w; uint16_t e[8]; } t;
+                t.w = col0 < row ? *(const uint4*) (kb + (int64_t) jr * row + col0) : uint4{0u, 0u, 0u, 0u};
+                sc[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(t.v, qf[s], sc[u], 0, 0, 0);
+                if (s < NV / 2)
+                {
+                    #pragma unroll
+                    for (int e = 0; e < 8; ++e) vt[(col0 + e) * LM_VS + u * 16 + c] = t.e[e];
+                }
+            }
+        }
+        __syncthreads();
+        float mx = -INFINITY;
+        #pragma unroll
+        for (int u = 0; u < 2; ++u)
+        {
+            #pragma unroll
+            for (int i = 0; i < 4; ++i)
+            {
+                const bool ok = j0 + u * 16 + g * 4 + i < k_end;
+                sc[u][i] = ok ? sc[u][i] * scale : -INFINITY;
+                mx = fmaxf(mx, sc[u][i]);
+            }
+        }
+        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));                    // finite: key j0 is inside the split
+        const float mn = fmaxf(m, mx);
+        const float corr = expf(m - mn);
+        m = mn;
+        float sum = 0.f;
+        #pragma unroll
+        for (int u = 0; u < 2; ++u)
+        {
+            #pragma unroll
+            for (int i = 0; i < 4; ++i) { sc[u][i] = expf(sc[u][i] - mn); sum += sc[u][i]; }       // masked: exp(-inf) = 0
+        }
+        l = l * corr + sum;
+        bf16x8 pb;
+        #pragma unroll
+        for (int i = 0; i < 4; ++i) { pb[i] = (__bf16) sc[0][i]; pb[4 + i] = (__bf16) sc[1][i]; }
+        #pragma unroll
+        for (int t = 0; t < NV; ++t)
+        {
+            acc[t] *= corr;
+            union { bf16x8 v; bf16x4 h[2]; } va;
+            va.h[0] = *(const bf16x4*) (vt + (t * 16 + c) * LM_VS + g * 4);
+            va.h[1] = *(const bf16x4*) (vt + (t * 16 + c) * LM_VS + 16 + g * 4);
+            acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va.v, pb, acc[t], 0, 0, 0);
+        }
+    }
+    l += __shfl_xor(l, 16, 64);
+    l += __shfl_xor(l, 32, 64);
+    if (!head_ok) return;
+    if (g == 0) { part_ml[pidx * 2] = m; part_ml[pidx * 2 + 1] = l; }
+    float* po = part_o + pidx * (NV * 16);
+    #pragma unroll
+    for (int t = 0; t < NV; ++t) *(f32x4*) (po + t * 16 + g * 4) = acc[t];          // acc[t][i] = latent column t*16 + 4g + i of head c
+}
+
+// o_lat[n][h] = sum_s e^(m_s - M) O_s / (sum_s e^(m_s - M) l_s + e^(sink - M)), M = max(m_s, sink); splits without keys are skipped
+__global__ __launch_bounds__(128) void latent_decode_merge_kernel(bf16_t* __restrict__ o_lat, int64_t o_row, int64_t o_head, const float* __restrict__ part_o,
+                                                                  const float* __restrict__ part_ml, const float* __restrict__ sink, int splits, int heads, int rank, int rp)
+{
+    const int n = blockIdx.x, h = blockIdx.y;
+    float M = sink ? sink[h] : -INFINITY;
+    for (int s = 0; s < splits; ++s) M = fmaxf(M, part_ml[(((int64_t) n * splits + s) * heads + h) * 2]);
+    float L = sink ? expf(sink[h] - M) : 0.f;
+    for (int s = 0; s < splits; ++s)
+    {
+        const float* ml = part_ml + (((int64_t) n * splits + s) * heads + h) * 2;
+        if (ml[1] > 0.f) L += ml[1] * expf(ml[0] - M);
+    }
+    const float inv = L > 0.f ? 1.0f / L : 0.f;
+    for (int col = threadIdx.x; col < rank; col += 128)
+    {
+        float a = 0.f;
+        for (int s = 0; s < splits; ++s)
+        {
+            const int64_t pi = ((int64_t) n * splits + s) * heads + h;
+            if (part_ml[pi * 2 + 1] > 0.f) a += part_o[pi * rp + col] * expf(part_ml[pi * 2] - M);
+        }
+        o_lat[(int64_t) n * o_row + (int64_t) h * o_head + col] = from_f<bf16_t>(a * inv);
+    }
+}
+
+extern "C" int exl3_mix_latent_decode_mfma_scratch(int n, int heads, int rank, int splits, int64_t* floats)
+{
+    MIX_CHECK(floats && n >= 0 && heads > 0 && rank > 0 && rank <= 512 && splits > 0, "mix_latent_decode_mfma_scratch: bad arguments");
+    const int rp = rank <= 128 ? 128 : (rank <= 256 ? 256 : 512);
+    *floats = (int64_t) n * splits * heads * (rp + 2);
+    return EXL3_MIX_OK;
+}
+
+extern "C" int exl3_mix_latent_decode_mfma(void* o_lat, int64_t o_row, int64_t o_head, const void* q_lat, int64_t ql_row, int64_t ql_head, const void* q, int64_t q_ld,
+                                           const void* ring, const float* sink, const int32_t* slots, const int32_t* len_after, float* scratch, int splits,
+                                           int n, int heads, int dim, int rot_dim, int rank, float scale, int window, void* stream)
+{
+    MIX_CHECK(o_lat && q_lat && q && ring && slots && len_after && scratch, "mix_latent_decode_mfma: null pointer");
+    MIX_CHECK(n >= 0 && n <= 65535 && heads > 0 && dim >= 0 && window > 0 && splits > 0 && splits <= 65535, "mix_latent_decode_mfma: bad sizes");
+    MIX_CHECK(rank > 0 && rank <= 512 && rank % 8 == 0 && rot_dim >= 0 && rot_dim % 8 == 0, "mix_latent_decode_mfma: rank %d and rot_dim %d must be multiples of 8, rank <= 512", rank, rot_dim);
+    const int nv = rank <= 128 ? 8 : (rank <= 256 ? 16 : 32);
+    MIX_CHECK(rank + rot_dim <= (nv / 2 + 2) * 32, "mix_latent_decode_mfma: rot_dim %d too large beside rank %d", rot_dim, rank);
+    MIX_CHECK((uintptr_t) ring % 16 == 0 && q_ld >= (int64_t) heads * (dim + rot_dim), "mix_latent_decode_mfma: the ring must be 16-byte aligned");
+    if (n == 0) return EXL3_MIX_OK;
+    const int keys_per_split = (((window + splits - 1) / splits) + LM_KEYS - 1) / LM_KEYS * LM_KEYS;
+    const int rp = nv * 16;
+    float* part_o = scratch;
+    float* part_ml = scratch + (int64_t) n * splits * heads * rp;
+    const dim3 grid(splits, (heads + 15) / 16, n);
+    #define LM_LAUNCH(NVV) hipLaunchKernelGGL((latent_decode_mfma_kernel<NVV, NVV / 2 + 2>), grid, dim3(64), 0, (hipStream_t) stream, part_o, part_ml, (const bf16_t*) q_lat, ql_row, \
+                                              ql_head, (const bf16_t*) q, q_ld, (const bf16_t*) ring, slots, len_after, heads, dim, rot_dim, rank, scale, window, keys_per_split)
+    if (nv == 8) LM_LAUNCH(8); else if (nv == 16) LM_LAUNCH(16); else LM_LAUNCH(32);
+    #undef LM_LAUNCH
+    if (int rc = mix_check_launch("mix_latent_decode_mfma")) return rc;
+    hipLaunchKernelGGL(latent_decode_merge_kernel, dim3(n, heads), dim3(128), 0, (hipStream_t) stream, (bf16_t*) o_lat, o_row, o_head, part_o, part_ml, sink, splits, heads, rank, rp);
+    return mix_check_launch("mix_latent_decode_mfma (merge)");
 }

@@ -259,7 +259,8 @@ def absorbed_reference(q_lat, q_rot, ring_rows, scale, sink):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("H,d,r,rank,W", [(2, 8, 8, 24, 5), (3, 16, 4, 130, 64), (1, 4, 16, 520, 300), (2, 8, 6, 37, 1)])
+@pytest.mark.parametrize("H,d,r,rank,W", [(2, 8, 8, 24, 5), (3, 16, 4, 130, 64), (1, 4, 16, 520, 300), (2, 8, 6, 37, 1), (3, 16, 16, 256, 64), (18, 8, 8, 136, 40),
+                                          (2, 8, 64, 512, 70), (16, 8, 24, 104, 33)])
 def test_latent_cache_kernels_window_edges(gpu, dtype, H, d, r, rank, W):
     """latent_prep + latent_decode alone, with one key made to stand out: the key that is W - 1 tokens back is seen, the one W back is not, in a
     ring that has wrapped; rows of the cache that a sequence has not written hold NaN and must not be read."""
@@ -308,13 +309,16 @@ def test_latent_cache_kernels_window_edges(gpu, dtype, H, d, r, rank, W):
             q_lat = torch.randn(H, 1, rank, generator=g) * 0.1 + 4.0 * c[edge].float() / (c[edge].norm() ** 2).float() * rank ** 0.5
             q_lat = q_lat.to(dtype)
             o_lat = torch.full((H, 1, rank), float("nan"), dtype=dtype, device=gpu)
+            kernels = [False, True] if mix_ops.latent_mfma_ok(dtype, rank, r) else [False]           # lane-per-key kernel, matrix-core kernel
             for sk in (None, sink):
-                mix_ops.latent_decode(o_lat, q_lat.to(gpu), q1, ring, None if sk is None else sk.to(gpu), sl, la, d, r, 0.9)
-                lo = max(0, t - W + 1)
-                want = torch.stack([absorbed_reference(q_lat[h, 0].to(F64), qr[t, h], rows[lo: t + 1], 0.9, None if sk is None else sk[h].to(F64)) for h in range(H)])
-                assert rel(o_lat[:, 0], want) < TOL[dtype], (t, edge, sk is None)
-                if edge >= lo and W > 1 and sk is None:
-                    assert rel(o_lat[:, 0], c[edge].expand(H, rank)) < 0.2          # the test's premise: that key dominates when it is inside
+                for mfma in kernels:
+                    o_lat.fill_(float("nan"))
+                    mix_ops.latent_decode(o_lat, q_lat.to(gpu), q1, ring, None if sk is None else sk.to(gpu), sl, la, d, r, 0.9, mfma=mfma)
+                    lo = max(0, t - W + 1)
+                    want = torch.stack([absorbed_reference(q_lat[h, 0].to(F64), qr[t, h], rows[lo: t + 1], 0.9, None if sk is None else sk[h].to(F64)) for h in range(H)])
+                    assert rel(o_lat[:, 0], want) < TOL[dtype], (t, edge, sk is None, mfma)
+                    if edge >= lo and W > 1 and sk is None:
+                        assert rel(o_lat[:, 0], c[edge].expand(H, rank)) < 0.2          # the test's premise: that key dominates when it is inside
     assert torch.isnan(ring[:slot]).all() and not torch.isnan(ring[slot]).any()
 
 
@@ -567,3 +571,34 @@ def test_trace_replay_writes_the_wanted_logits(gpu, zoo, tmp_path):
     assert not os.path.exists(os.path.join(str(tmp_path), "2.f32"))
     assert rel(rd(3), ra[11:12]) < TOL[torch.float32]
     assert sess.cache.in_use() == 0
+
+
+@pytest.mark.parametrize("H,r,rank,W,lens", [(5, 16, 64, 100, [3, 100, 57, 1]), (33, 8, 128, 300, [299, 301, 64]), (16, 64, 512, 129, [129, 40]), (4, 0, 200, 77, [500, 76])])
+def test_matrix_core_latent_decode_batches_and_splits(gpu, H, r, rank, W, lens):
+    """The matrix-core decode kernel over a batch of sequences of unequal length (shorter than, equal to and longer than the window, so rings are part
+    filled, exactly full and wrapped), with every number of key splits from one to more than there are key tiles, against the float64 form."""
+    from exllamav3_amd import mix_ops
+    g = torch.Generator().manual_seed(rank + W)
+    B, row, d = len(lens), rank + r, 8
+    ring = torch.full((B + 2, W, row), float("nan"), dtype=torch.bfloat16, device=gpu)
+    slots = [B + 1 - i for i in range(B)]
+    rows = []
+    for b, L in enumerate(lens):
+        cnt = min(L, W)
+        data = torch.randn(cnt, row, generator=g).to(torch.bfloat16)
+        ring[slots[b], :cnt] = data.to(gpu)
+        rows.append(data.to(F64))
+    q_lat = (torch.randn(H, B, rank, generator=g) * 0.3).to(torch.bfloat16)
+    q = torch.randn(B, H * (d + r), generator=g).to(torch.bfloat16)
+    sink = torch.randn(H, generator=g)
+    for sk in (None, sink):
+        want = torch.stack([torch.stack([absorbed_reference(q_lat[h, b].to(F64), q[b].view(H, d + r)[h, d:].to(F64), rows[b], 0.2, None if sk is None else sk[h].to(F64))
+                                         for b in range(B)]) for h in range(H)])
+        for target in (1, 7, 64, 4096):
+            mix_ops.LATENT_MFMA_TARGET_WAVES, keep = target, mix_ops.LATENT_MFMA_TARGET_WAVES
+            try:
+                o = torch.full((H, B, rank), float("nan"), dtype=torch.bfloat16, device=gpu)
+                mix_ops.latent_decode(o, q_lat.to(gpu), q.to(gpu), ring, None if sk is None else sk.to(gpu), mk(gpu, slots), mk(gpu, lens), d, r, 0.2, mfma=True)
+            finally:
+                mix_ops.LATENT_MFMA_TARGET_WAVES = keep
+            assert rel(o, want) < TOL[torch.bfloat16], (sk is None, target)
