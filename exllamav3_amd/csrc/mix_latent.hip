@@ -168,7 +168,7 @@ template <int NV, int KD>
 __global__ __launch_bounds__(64) void latent_decode_mfma_kernel(float* __restrict__ part_o, float* __restrict__ part_ml, const bf16_t* __restrict__ q_lat, int64_t ql_row,
                                                                  int64_t ql_head, const bf16_t* __restrict__ q, int64_t q_ld, const bf16_t* __restrict__ ring,
                                                                  const int32_t* __restrict__ slots, const int32_t* __restrict__ len_after,
-                                                                 int heads, int dim, int rot_dim, int rank, float scale, int window, int keys_per_split)
+                                                                 int heads, int dim, int rot_dim, int rank, float scale, int window, int keys_per_split, int q_vec)
 {
     __shared__ __attribute__((aligned(16))) uint16_t vt[NV * 16 * LM_VS];        // [latent column][key of the tile]
     const int sp = blockIdx.x, hg = blockIdx.y, n = blockIdx.z, splits = gridDim.x;
@@ -189,15 +189,16 @@ __global__ __launch_bounds__(64) void latent_decode_mfma_kernel(float* __restric
     #pragma unroll
     for (int s = 0; s < KD; ++s)
     {
-        union { bf16x8 v; uint16_t u[8]; } t;
-        #pragma unroll
-        for (int e = 0; e < 8; ++e)
+        union { bf16x8 v; uint4 w; uint16_t u[8]; } t;
+        const int c0 = s * 32 + g * 8;                            // rank and row are multiples of 8: the group lies in one part of the query or beyond it
+        const bf16_t* src = c0 < rank ? q_lat + (int64_t) n * ql_row + (int64_t) head * ql_head + c0
+                                      : q + (int64_t) n * q_ld + (int64_t) head * (dim + rot_dim) + dim + (c0 - rank);
+        if (!head_ok || c0 >= row) t.w = uint4{0u, 0u, 0u, 0u};
+        else if (q_vec) t.w = *(const uint4*) src;                // 16-byte groups (host-checked alignment)
+        else
         {
-            const int col = s * 32 + g * 8 + e;
-            uint16_t x = 0;
-            if (head_ok && col < rank) x = q_lat[(int64_t) n * ql_row + (int64_t) head * ql_head + col].u;
-            else if (head_ok && col < row) x = q[(int64_t) n * q_ld + (int64_t) head * (dim + rot_dim) + dim + (col - rank)].u;
-            t.u[e] = x;
+            #pragma unroll
+            for (int e = 0; e < 8; ++e) t.u[e] = src[e].u;
         }
         qf[s] = t.v;
     }
@@ -207,6 +208,17 @@ __global__ __launch_bounds__(64) void latent_decode_mfma_kernel(float* __restric
     for (int t = 0; t < NV; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
     for (int j0 = k_begin; j0 < k_end; j0 += LM_KEYS)
     {
+        // all of the tile's rows first (2 x KD independent 16-byte loads in flight), then the products
+        union kreg { bf16x8 v; uint4 w; uint16_t e[8]; };
+        kreg kf[2][KD];
+        #pragma unroll
+        for (int u = 0; u < 2; ++u)
+        {
+            const int jr = min(j0 + u * 16 + c, count - 1);       // rows past the split are read (they exist) and masked below
+            const bf16_t* kr = kb + (int64_t) jr * row + g * 8;   // row is a multiple of 8: a group of 8 columns is inside the row or outside
+            #pragma unroll
+            for (int s = 0; s < KD; ++s) kf[u][s].w = s * 32 + g * 8 < row ? *(const uint4*) (kr + s * 32) : uint4{0u, 0u, 0u, 0u};
+        }
         __syncthreads();                                           // one wave: the previous tile's operand reads are over
         f32x4 sc[2] = {f32x4{0.f, 0.f, 0.f, 0.f}, f32x4{0.f, 0.f, 0.f, 0.f}};
         #pragma unroll
@@ -215,15 +227,11 @@ __global__ __launch_bounds__(64) void latent_decode_mfma_kernel(float* __restric
             #pragma unroll
             for (int u = 0; u < 2; ++u)
             {
-                const int jr = min(j0 + u * 16 + c, count - 1);   // rows past the split are read (they exist) and masked below
-                const int col0 = s * 32 + g * 8;                  // row is a multiple of 8: a group of 8 columns is inside the row or outside
-                union { bf16x8 v; uint4 w; uint16_t e[8]; } t;
-                t.w = col0 < row ? *(const uint4*) (kb + (int64_t) jr * row + col0) : uint4{0u, 0u, 0u, 0u};
-                sc[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(t.v, qf[s], sc[u], 0, 0, 0);
+                sc[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[u][s].v, qf[s], sc[u], 0, 0, 0);
                 if (s < NV / 2)
                 {
                     #pragma unroll
-                    for (int e = 0; e < 8; ++e) vt[(col0 + e) * LM_VS + u * 16 + c] = t.e[e];
+                    for (int e = 0; e < 8; ++e) vt[(s * 32 + g * 8 + e) * LM_VS + u * 16 + c] = kf[u][s].e[e];
                 }
             }
         }
@@ -275,27 +283,43 @@ __global__ __launch_bounds__(64) void latent_decode_mfma_kernel(float* __restric
     for (int t = 0; t < NV; ++t) *(f32x4*) (po + t * 16 + g * 4) = acc[t];          // acc[t][i] = latent column t*16 + 4g + i of head c
 }
 
-// o_lat[n][h] = sum_s e^(m_s - M) O_s / (sum_s e^(m_s - M) l_s + e^(sink - M)), M = max(m_s, sink); splits without keys are skipped
+// o_lat[n][h] = sum_s e^(m_s - M) O_s / (sum_s e^(m_s - M) l_s + e^(sink - M)), M = max(m_s, sink); splits without keys weigh nothing (their sums are
+// never read into the result: unwritten scratch may hold anything).  The splits' weights are computed once into LDS; the sum over splits then has
+// independent loads.
 __global__ __launch_bounds__(128) void latent_decode_merge_kernel(bf16_t* __restrict__ o_lat, int64_t o_row, int64_t o_head, const float* __restrict__ part_o,
                                                                   const float* __restrict__ part_ml, const float* __restrict__ sink, int splits, int heads, int rank, int rp)
 {
+    extern __shared__ float wsm[];                              // [splits]
+    __shared__ float red[2];
     const int n = blockIdx.x, h = blockIdx.y;
-    float M = sink ? sink[h] : -INFINITY;
-    for (int s = 0; s < splits; ++s) M = fmaxf(M, part_ml[(((int64_t) n * splits + s) * heads + h) * 2]);
-    float L = sink ? expf(sink[h] - M) : 0.f;
-    for (int s = 0; s < splits; ++s)
+    const float* ml = part_ml + ((int64_t) n * splits * heads + h) * 2;         // split s at ml + s * heads * 2
+    const float* po = part_o + ((int64_t) n * splits * heads + h) * rp;         // split s at po + s * heads * rp
+    const float sk = sink ? sink[h] : -INFINITY;
+    float mloc = -INFINITY;
+    for (int s = threadIdx.x; s < splits; s += 128) mloc = fmaxf(mloc, ml[(int64_t) s * heads * 2]);
+    mloc = wave_max(mloc);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = mloc;
+    __syncthreads();
+    const float M = fmaxf(fmaxf(red[0], red[1]), sk);
+    float lloc = 0.f;
+    for (int s = threadIdx.x; s < splits; s += 128)
     {
-        const float* ml = part_ml + (((int64_t) n * splits + s) * heads + h) * 2;
-        if (ml[1] > 0.f) L += ml[1] * expf(ml[0] - M);
+        const float ls = ml[(int64_t) s * heads * 2 + 1];
+        const float w = ls > 0.f ? expf(ml[(int64_t) s * heads * 2] - M) : 0.f;
+        wsm[s] = w;
+        lloc += w * ls;
     }
+    lloc = block_sum<2>(lloc, red);                             // its barriers also publish wsm
+    const float L = lloc + (sink ? expf(sk - M) : 0.f);
     const float inv = L > 0.f ? 1.0f / L : 0.f;
     for (int col = threadIdx.x; col < rank; col += 128)
     {
         float a = 0.f;
+        #pragma unroll 8
         for (int s = 0; s < splits; ++s)
         {
-            const int64_t pi = ((int64_t) n * splits + s) * heads + h;
-            if (part_ml[pi * 2 + 1] > 0.f) a += part_o[pi * rp + col] * expf(part_ml[pi * 2] - M);
+            const float w = wsm[s], v = po[(int64_t) s * heads * rp + col];
+            a += w != 0.f ? w * v : 0.f;
         }
         o_lat[(int64_t) n * o_row + (int64_t) h * o_head + col] = from_f<bf16_t>(a * inv);
     }
@@ -322,14 +346,15 @@ extern "C" int exl3_mix_latent_decode_mfma(void* o_lat, int64_t o_row, int64_t o
     if (n == 0) return EXL3_MIX_OK;
     const int keys_per_split = (((window + splits - 1) / splits) + LM_KEYS - 1) / LM_KEYS * LM_KEYS;
     const int rp = nv * 16;
+    const int q_vec = (uintptr_t) q_lat % 16 == 0 && ql_row % 8 == 0 && ql_head % 8 == 0 && (uintptr_t) q % 16 == 0 && q_ld % 8 == 0 && dim % 8 == 0;
     float* part_o = scratch;
     float* part_ml = scratch + (int64_t) n * splits * heads * rp;
     const dim3 grid(splits, (heads + 15) / 16, n);
     #define LM_LAUNCH(NVV) hipLaunchKernelGGL((latent_decode_mfma_kernel<NVV, NVV / 2 + 2>), grid, dim3(64), 0, (hipStream_t) stream, part_o, part_ml, (const bf16_t*) q_lat, ql_row, \
-                                              ql_head, (const bf16_t*) q, q_ld, (const bf16_t*) ring, slots, len_after, heads, dim, rot_dim, rank, scale, window, keys_per_split)
+                                              ql_head, (const bf16_t*) q, q_ld, (const bf16_t*) ring, slots, len_after, heads, dim, rot_dim, rank, scale, window, keys_per_split, q_vec)
     if (nv == 8) LM_LAUNCH(8); else if (nv == 16) LM_LAUNCH(16); else LM_LAUNCH(32);
     #undef LM_LAUNCH
     if (int rc = mix_check_launch("mix_latent_decode_mfma")) return rc;
-    hipLaunchKernelGGL(latent_decode_merge_kernel, dim3(n, heads), dim3(128), 0, (hipStream_t) stream, (bf16_t*) o_lat, o_row, o_head, part_o, part_ml, sink, splits, heads, rank, rp);
+    hipLaunchKernelGGL(latent_decode_merge_kernel, dim3(n, heads), dim3(128), (size_t) splits * sizeof(float), (hipStream_t) stream, (bf16_t*) o_lat, o_row, o_head, part_o, part_ml, sink, splits, heads, rank, rp);
     return mix_check_launch("mix_latent_decode_mfma (merge)");
 }

@@ -70,28 +70,53 @@ __global__ __launch_bounds__(ROW_THREADS) void dyn_tanh_rows_kernel(T* __restric
     for (int i = threadIdx.x; i < width; i += ROW_THREADS) h[(int64_t) n * width + i] = from_f<T>(tanhf(alpha * xr[i]) * w[i] + b[i]);
 }
 
-// plain activations: 0 = relu(z)^2, 1 = gelu (tanh form), 2 = silu
-template <typename T>
-__global__ __launch_bounds__(256) void act_kernel(T* __restrict__ out, const T* __restrict__ z, int64_t z_ld, int ff, int kind)
+// plain activations: 0 = relu(z)^2, 1 = gelu (tanh form), 2 = silu.  A thread takes VN consecutive elements (16 bytes) when the rows allow it.
+template <typename T> struct rvec;
+template <> struct rvec<bf16_t> { static constexpr int N = 8; };
+template <> struct rvec<float> { static constexpr int N = 4; };
+
+__device__ __forceinline__ float act_f(float v, int kind)
 {
-    const int n = blockIdx.y;
-    const int i = blockIdx.x * 256 + threadIdx.x;
-    if (i >= ff) return;
-    const float v = to_f(z[(int64_t) n * z_ld + i]);
-    float r;
-    if (kind == 0) { const float t = fmaxf(v, 0.f); r = t * t; }
-    else if (kind == 1) r = gelu_tanh_f(v);
-    else r = silu_f(v);
-    out[(int64_t) n * ff + i] = from_f<T>(r);
+    if (kind == 0) { const float t = fmaxf(v, 0.f); return t * t; }
+    if (kind == 1) return gelu_tanh_f(v);
+    return silu_f(v);
 }
 
-template <typename T>
+template <typename T, bool VEC>
+__global__ __launch_bounds__(256) void act_kernel(T* __restrict__ out, const T* __restrict__ z, int64_t z_ld, int ff, int kind)
+{
+    constexpr int VN = VEC ? rvec<T>::N : 1;
+    const int n = blockIdx.y;
+    const int i = (blockIdx.x * 256 + threadIdx.x) * VN;
+    if (i >= ff) return;
+    if (VEC)
+    {
+        union { uint4 v; T e[rvec<T>::N]; } a, o;
+        a.v = *(const uint4*) (z + (int64_t) n * z_ld + i);
+        #pragma unroll
+        for (int e = 0; e < rvec<T>::N; ++e) o.e[e] = from_f<T>(act_f(to_f(a.e[e]), kind));
+        *(uint4*) (out + (int64_t) n * ff + i) = o.v;
+    }
+    else out[(int64_t) n * ff + i] = from_f<T>(act_f(to_f(z[(int64_t) n * z_ld + i]), kind));
+}
+
+template <typename T, bool VEC>
 __global__ __launch_bounds__(256) void glu_act_kernel(T* __restrict__ out, const T* __restrict__ g, int64_t g_ld, const T* __restrict__ u, int64_t u_ld, int ff, int kind, float limit)
 {
+    constexpr int VN = VEC ? rvec<T>::N : 1;
     const int n = blockIdx.y;
-    const int i = blockIdx.x * 256 + threadIdx.x;
+    const int i = (blockIdx.x * 256 + threadIdx.x) * VN;
     if (i >= ff) return;
-    out[(int64_t) n * ff + i] = from_f<T>(glu_act_f(to_f(g[(int64_t) n * g_ld + i]), to_f(u[(int64_t) n * u_ld + i]), kind, limit));
+    if (VEC)
+    {
+        union { uint4 v; T e[rvec<T>::N]; } a, b, o;
+        a.v = *(const uint4*) (g + (int64_t) n * g_ld + i);
+        b.v = *(const uint4*) (u + (int64_t) n * u_ld + i);
+        #pragma unroll
+        for (int e = 0; e < rvec<T>::N; ++e) o.e[e] = from_f<T>(glu_act_f(to_f(a.e[e]), to_f(b.e[e]), kind, limit));
+        *(uint4*) (out + (int64_t) n * ff + i) = o.v;
+    }
+    else out[(int64_t) n * ff + i] = from_f<T>(glu_act_f(to_f(g[(int64_t) n * g_ld + i]), to_f(u[(int64_t) n * u_ld + i]), kind, limit));
 }
 
 // out[n][j] = gelu_tanh(gate[n][j]) * table[tokens[n]][col0 + j]
@@ -183,11 +208,17 @@ extern "C" int exl3_mix_dyn_tanh_rows(void* h, const float* x, const int32_t* ro
 extern "C" int exl3_mix_act(void* out, const void* z, int64_t z_ld, int n, int ff, int kind, int dtype, void* stream)
 {
     MIX_CHECK(out && z && n >= 0 && n <= 65535 * 1024 && ff > 0 && z_ld >= ff && kind >= 0 && kind <= 2, "mix_act: bad arguments");
+    const int vn = dtype == EXL3_MIX_BF16 ? 8 : 4;
+    const bool vec = ff % vn == 0 && z_ld % vn == 0 && (uintptr_t) out % 16 == 0 && (uintptr_t) z % 16 == 0;
     for (int r0 = 0; r0 < n; r0 += 65535)
     {
         const int rows = n - r0 < 65535 ? n - r0 : 65535;
-        MIX_DISPATCH_T(dtype, hipLaunchKernelGGL(act_kernel<T>, dim3((ff + 255) / 256, rows), dim3(256), 0, (hipStream_t) stream, (T*) out + (int64_t) r0 * ff,
-                                                 (const T*) z + (int64_t) r0 * z_ld, z_ld, ff, kind));
+        if (vec)
+            MIX_DISPATCH_T(dtype, hipLaunchKernelGGL((act_kernel<T, true>), dim3((ff / vn + 255) / 256, rows), dim3(256), 0, (hipStream_t) stream, (T*) out + (int64_t) r0 * ff,
+                                                     (const T*) z + (int64_t) r0 * z_ld, z_ld, ff, kind));
+        else
+            MIX_DISPATCH_T(dtype, hipLaunchKernelGGL((act_kernel<T, false>), dim3((ff + 255) / 256, rows), dim3(256), 0, (hipStream_t) stream, (T*) out + (int64_t) r0 * ff,
+                                                     (const T*) z + (int64_t) r0 * z_ld, z_ld, ff, kind));
     }
     return mix_check_launch("mix_act");
 }
@@ -195,11 +226,17 @@ extern "C" int exl3_mix_act(void* out, const void* z, int64_t z_ld, int n, int f
 extern "C" int exl3_mix_glu_act(void* out, const void* g, int64_t g_ld, const void* u, int64_t u_ld, int n, int ff, int kind, float limit, int dtype, void* stream)
 {
     MIX_CHECK(out && g && u && n >= 0 && ff > 0 && g_ld >= ff && u_ld >= ff && kind >= 0 && kind <= 1, "mix_glu_act: bad arguments");
+    const int vn = dtype == EXL3_MIX_BF16 ? 8 : 4;
+    const bool vec = ff % vn == 0 && g_ld % vn == 0 && u_ld % vn == 0 && (uintptr_t) out % 16 == 0 && (uintptr_t) g % 16 == 0 && (uintptr_t) u % 16 == 0;
     for (int r0 = 0; r0 < n; r0 += 65535)
     {
         const int rows = n - r0 < 65535 ? n - r0 : 65535;
-        MIX_DISPATCH_T(dtype, hipLaunchKernelGGL(glu_act_kernel<T>, dim3((ff + 255) / 256, rows), dim3(256), 0, (hipStream_t) stream, (T*) out + (int64_t) r0 * ff,
-                                                 (const T*) g + (int64_t) r0 * g_ld, g_ld, (const T*) u + (int64_t) r0 * u_ld, u_ld, ff, kind, limit));
+        if (vec)
+            MIX_DISPATCH_T(dtype, hipLaunchKernelGGL((glu_act_kernel<T, true>), dim3((ff / vn + 255) / 256, rows), dim3(256), 0, (hipStream_t) stream, (T*) out + (int64_t) r0 * ff,
+                                                     (const T*) g + (int64_t) r0 * g_ld, g_ld, (const T*) u + (int64_t) r0 * u_ld, u_ld, ff, kind, limit));
+        else
+            MIX_DISPATCH_T(dtype, hipLaunchKernelGGL((glu_act_kernel<T, false>), dim3((ff + 255) / 256, rows), dim3(256), 0, (hipStream_t) stream, (T*) out + (int64_t) r0 * ff,
+                                                     (const T*) g + (int64_t) r0 * g_ld, g_ld, (const T*) u + (int64_t) r0 * u_ld, u_ld, ff, kind, limit));
     }
     return mix_check_launch("mix_glu_act");
 }

@@ -21,8 +21,8 @@ KINDS = [("latent_attention_2", "dense"), ("latent_attention", "moe")]
 YARN = {"factor": 4.0, "original": 4096, "fast": 32.0, "slow": 1.0}
 
 
-def synth(size_name: str, kinds, vocab=32000, seed=0, device="cuda:0"):
-    size, lt = SIZES[size_name], LATENT[size_name]
+def synth(size: dict, lt: dict, kinds, vocab=32000, seed=0, device="cuda:0", loop=None):
+    """Random Zagilorn weights and their config: size = width / ff / window / moe (experts, top, expert ff), lt = the latent-attention shape; loop = (start, stop, times)."""
     g = torch.Generator(device=device).manual_seed(seed)
     w, t, layers = size["width"], {}, []
 
@@ -59,13 +59,16 @@ def synth(size_name: str, kinds, vocab=32000, seed=0, device="cuda:0"):
         lin(p + "side.gate", lt["side"], w); lin(p + "side.proj", w, lt["side"]); vec(p + "side.norm", w, 1.0)
         layers.append({"type": mix, "mixer": mixer, "mlp": mlp})
     cfg = {"architecture": "Zagilorn", "vocab": vocab, "width": w, "norm": {"eps": 1e-5}, "logit_scale": 1.0, "token_side": {"dim": lt["side"]}, "layers": layers}
+    if loop:
+        lin("loop.in", w, 2 * w, 1.4)
+        cfg["loop"] = {"start": loop[0], "stop": loop[1], "times": loop[2]}
     return cfg, TensorDict(t)
 
 
 def _make(size_name):
     def make(size, kind, reps, dev):
         from .zagilorn import ZagilornModel
-        cfg, td = synth(size_name, [kind] * reps, device=dev)
+        cfg, td = synth(size, LATENT[size_name], [kind] * reps, device=dev)
         return ZagilornModel(cfg, td, device=dev, dtype=torch.bfloat16)
     return make
 
@@ -108,8 +111,8 @@ def latent_kernel_legs(size_name: str, prompt: int, ctx: int, dev):
         e = hbm(by, t)
         e["tflops"] = bs * H * min(ctx, W) * (row + rank) * 2.0 / t / 1e12
         out[f"latent_decode_bs{bs}"] = e
-        dkd, ck1, pd = rnd(bs, row), torch.empty((bs, row), dtype=bf, device=dev), i32([ctx - 1] * bs)
-        t = _time(lambda: mix_ops.latent_prep(ck1, ring, dkd, nw, qd, torch.arange(bs, dtype=torch.int32, device=dev), pd, sld, lad, freq, mag, 1e-5, H, d, r, rank), 50)
+        dkd, ck1, pd, sq = rnd(bs, row), torch.empty((bs, row), dtype=bf, device=dev), i32([ctx - 1] * bs), torch.arange(bs, dtype=torch.int32, device=dev)
+        t = _time(lambda: mix_ops.latent_prep(ck1, ring, dkd, nw, qd, sq, pd, sld, lad, freq, mag, 1e-5, H, d, r, rank), 50)
         out[f"latent_prep_bs{bs}"] = {"us": t * 1e6}
     x, y, nb, h = torch.randn(n, w, device=dev), rnd(n, w), torch.zeros(w, device=dev), torch.empty((n, w), dtype=bf, device=dev)
     nw2 = torch.ones(w, device=dev)

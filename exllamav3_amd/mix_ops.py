@@ -358,8 +358,8 @@ def latent_fill_k(k: torch.Tensor, ckr: torch.Tensor, heads: int, dim: int, rot_
     _check(_lib.mixlib().exl3_mix_latent_fill_k(_p(k), _view(k, heads * (dim + rot_dim), "k"), _p(ckr), n, heads, dim, rot_dim, rank, code(k.dtype), _stream(k)))
 
 
-# decode steps on the matrix cores: the cached rows of a sequence are split so that about this many waves are in flight
-LATENT_MFMA_TARGET_WAVES = 512
+# decode steps on the matrix cores: the cached rows of a sequence are split so that about this many one-wave workgroups are in flight (four fit a CU)
+LATENT_MFMA_TARGET_WAVES = 1024
 
 
 def latent_mfma_ok(dtype, rank: int, rot_dim: int) -> bool:

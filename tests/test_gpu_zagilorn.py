@@ -200,10 +200,11 @@ def test_residual_update_and_dyn_tanh(gpu, dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_activations_token_gate_heads_gate(gpu, dtype):
+@pytest.mark.parametrize("ff", [70, 72, 2056])                      # element by element, and 16 bytes per thread (one block, several blocks)
+def test_activations_token_gate_heads_gate(gpu, dtype, ff):
     from exllamav3_amd import mix_ops
     g = torch.Generator().manual_seed(4)
-    n, ff = 9, 70
+    n = 9
     z = (3 * torch.randn(n, 2 * ff, generator=g)).to(dtype)
     a, b = z[:, :ff].to(F64), z[:, ff:].to(F64)
     zd = z.to(gpu)
