@@ -10,7 +10,7 @@
 //                   caller up-projects with W_uv.  Scores, softmax and sums are the float32 row worker of mix_attn_row.cuh.
 //   latent_decode_mfma   the same on the matrix cores (bfloat16): all heads of a sequence score the SAME cached rows, so sixteen heads are the
 //                   sixteen columns of one MFMA tile and every cached row is read once per sixteen heads instead of once per head.  The keys of a
-//                   sequence are split over workgroups of one wave; a second kernel merges the partial sums (and adds the sink).
+//                   sequence are split over workgroups whose four waves share the rows' columns; a second kernel merges the partial sums (and adds the sink).
 #include "mix_common.cuh"
 #include "mix_attn_row.cuh"
 
@@ -151,91 +151,106 @@ extern "C" int exl3_mix_latent_decode(void* o_lat, int64_t o_row, int64_t o_head
 }
 
 // ---- decode on the matrix cores ---------------------------------------------------------------------------------------------------------------
-// One wave = one split of one sequence's cached rows x one group of 16 heads.  v_mfma_f32_16x16x32_bf16 operand lane (g = lane / 16, c = lane % 16)
-// holds row / column c and contraction slots 8g .. 8g+7; result lane (g, c) holds rows 4g .. 4g+3 of column c.
+// One workgroup of four waves = one split of one sequence's cached rows x one group of 16 heads.  v_mfma_f32_16x16x32_bf16 operand lane (g = lane / 16,
+// c = lane % 16) holds row / column c and contraction slots 8g .. 8g+7; result lane (g, c) holds rows 4g .. 4g+3 of column c.
 //   scores, transposed: S^T = K Q^T.  A = 16 cached rows (lane: row c, 16 bytes straight from the ring, no staging), B = the 16 heads' absorbed queries
 //   [q_lat | q_rot] (registers, loaded once).  A lane then holds the scores of ONE head, so the running maximum and sum are per-lane scalars.
 //   O^T = C^T P^T over tiles of 32 keys: the score registers of two 16-key tiles are the B operand as they stand when contraction slot (g, e) means key
 //   4g + e of the first tile (e < 4) or of the second (e >= 4); A = the latent columns of the same rows, transposed through LDS (the rows are in registers
 //   already: they were the A operands of the scores).
+// The four waves split the COLUMNS of the cached rows: wave w loads a quarter of every row (and one of the up to two 32-column steps behind the padded
+// latent), contributes that quarter's share of the scores -- summed through LDS in a fixed order, so every wave holds the same scores and repeats the few
+// softmax steps -- and owns the same quarter of the latent columns in the second product: a quarter of the accumulators, its own rows of C^T in LDS.
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 #define LM_KEYS 32
 #define LM_VS (LM_KEYS + 8)
+#define LM_WAVES 4
 
-template <int NV, int KD>
-__global__ __launch_bounds__(64) void latent_decode_mfma_kernel(float* __restrict__ part_o, float* __restrict__ part_ml, const bf16_t* __restrict__ q_lat, int64_t ql_row,
-                                                                 int64_t ql_head, const bf16_t* __restrict__ q, int64_t q_ld, const bf16_t* __restrict__ ring,
-                                                                 const int32_t* __restrict__ slots, const int32_t* __restrict__ len_after,
-                                                                 int heads, int dim, int rot_dim, int rank, float scale, int window, int keys_per_split, int q_vec)
+template <int NV>
+__global__ __launch_bounds__(64 * LM_WAVES) void latent_decode_mfma_kernel(float* __restrict__ part_o, float* __restrict__ part_ml, const bf16_t* __restrict__ q_lat,
+                                                                           int64_t ql_row, int64_t ql_head, const bf16_t* __restrict__ q, int64_t q_ld,
+                                                                           const bf16_t* __restrict__ ring, const int32_t* __restrict__ slots,
+                                                                           const int32_t* __restrict__ len_after, int heads, int dim, int rot_dim, int rank, float scale,
+                                                                           int window, int keys_per_split, int q_vec)
 {
-    __shared__ __attribute__((aligned(16))) uint16_t vt[NV * 16 * LM_VS];        // [latent column][key of the tile]
-    const int sp = blockIdx.x, hg = blockIdx.y, n = blockIdx.z, splits = gridDim.x;
-    const int lane = threadIdx.x, g = lane >> 4, c = lane & 15;
+    constexpr int KDW = NV / 8;                                 // 32-column steps of the padded latent per wave
+    constexpr int NVW = NV / 4;                                 // 16-column tiles of the latent per wave
+    constexpr int NS = KDW + 1;                                 // + one step behind the padded latent (columns NV * 16 + 32 w ..), empty for most waves
+    __shared__ __attribute__((aligned(16))) uint16_t vt[NV * 16 * LM_VS];        // [latent column][key of the tile]; wave w owns rows w * NV * 4 ..
+    __shared__ __attribute__((aligned(16))) float sp[LM_WAVES][2][64][4];         // the waves' shares of the scores
+    const int sp_i = blockIdx.x, hg = blockIdx.y, n = blockIdx.z, splits = gridDim.x;
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6, g = lane >> 4, c = lane & 15;
     const int count = min(len_after[n], window);
-    const int k_begin = sp * keys_per_split, k_end = min(count, k_begin + keys_per_split);
+    const int k_begin = sp_i * keys_per_split, k_end = min(count, k_begin + keys_per_split);
     const int row = rank + rot_dim;
     const bf16_t* kb = ring + (int64_t) slots[n] * window * row;
     const int head = hg * 16 + c;
     const bool head_ok = head < heads;
-    const int64_t pidx = ((int64_t) n * splits + sp) * heads + head;
+    const int64_t pidx = ((int64_t) n * splits + sp_i) * heads + head;
     if (k_begin >= k_end)
     {
-        if (head_ok && g == 0) { part_ml[pidx * 2] = -INFINITY; part_ml[pidx * 2 + 1] = 0.f; }
+        if (w == 0 && head_ok && g == 0) { part_ml[pidx * 2] = -INFINITY; part_ml[pidx * 2 + 1] = 0.f; }
         return;
     }
-    bf16x8 qf[KD];
+    // this wave's steps: first column of step i (rank and row are multiples of 8: a group of 8 columns lies in one part of the row or beyond it)
+    int col_of[NS];
     #pragma unroll
-    for (int s = 0; s < KD; ++s)
+    for (int i = 0; i < NS; ++i) col_of[i] = (i < KDW ? (w * KDW + i) * 32 : NV * 16 + w * 32) + g * 8;
+    bf16x8 qf[NS];
+    #pragma unroll
+    for (int i = 0; i < NS; ++i)
     {
-        union { bf16x8 v; uint4 w; uint16_t u[8]; } t;
-        const int c0 = s * 32 + g * 8;                            // rank and row are multiples of 8: the group lies in one part of the query or beyond it
+        union { bf16x8 v; uint4 x; uint16_t u[8]; } t;
+        const int c0 = col_of[i];
         const bf16_t* src = c0 < rank ? q_lat + (int64_t) n * ql_row + (int64_t) head * ql_head + c0
                                       : q + (int64_t) n * q_ld + (int64_t) head * (dim + rot_dim) + dim + (c0 - rank);
-        if (!head_ok || c0 >= row) t.w = uint4{0u, 0u, 0u, 0u};
-        else if (q_vec) t.w = *(const uint4*) src;                // 16-byte groups (host-checked alignment)
+        if (!head_ok || c0 >= row) t.x = uint4{0u, 0u, 0u, 0u};
+        else if (q_vec) t.x = *(const uint4*) src;                // 16-byte groups (host-checked alignment)
         else
         {
             #pragma unroll
             for (int e = 0; e < 8; ++e) t.u[e] = src[e].u;
         }
-        qf[s] = t.v;
+        qf[i] = t.v;
     }
     float m = -1e30f, l = 0.f;
-    f32x4 acc[NV];
+    f32x4 acc[NVW];
     #pragma unroll
-    for (int t = 0; t < NV; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int t = 0; t < NVW; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
     for (int j0 = k_begin; j0 < k_end; j0 += LM_KEYS)
     {
-        // all of the tile's rows first (2 x KD independent 16-byte loads in flight), then the products
-        union kreg { bf16x8 v; uint4 w; uint16_t e[8]; };
-        kreg kf[2][KD];
+        union kreg { bf16x8 v; uint4 x; uint16_t e[8]; };
+        kreg kf[2][NS];
         #pragma unroll
         for (int u = 0; u < 2; ++u)
         {
             const int jr = min(j0 + u * 16 + c, count - 1);       // rows past the split are read (they exist) and masked below
-            const bf16_t* kr = kb + (int64_t) jr * row + g * 8;   // row is a multiple of 8: a group of 8 columns is inside the row or outside
+            const bf16_t* kr = kb + (int64_t) jr * row;
             #pragma unroll
-            for (int s = 0; s < KD; ++s) kf[u][s].w = s * 32 + g * 8 < row ? *(const uint4*) (kr + s * 32) : uint4{0u, 0u, 0u, 0u};
+            for (int i = 0; i < NS; ++i) kf[u][i].x = col_of[i] < row ? *(const uint4*) (kr + col_of[i]) : uint4{0u, 0u, 0u, 0u};
         }
-        __syncthreads();                                           // one wave: the previous tile's operand reads are over
-        f32x4 sc[2] = {f32x4{0.f, 0.f, 0.f, 0.f}, f32x4{0.f, 0.f, 0.f, 0.f}};
+        __syncthreads();                                           // the previous tile's reads of sp and vt are over
         #pragma unroll
-        for (int s = 0; s < KD; ++s)
+        for (int u = 0; u < 2; ++u)
         {
+            f32x4 part = f32x4{0.f, 0.f, 0.f, 0.f};
             #pragma unroll
-            for (int u = 0; u < 2; ++u)
+            for (int i = 0; i < NS; ++i) part = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[u][i].v, qf[i], part, 0, 0, 0);
+            *(f32x4*) sp[w][u][lane] = part;
+            #pragma unroll
+            for (int i = 0; i < KDW; ++i)
             {
-                sc[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[u][s].v, qf[s], sc[u], 0, 0, 0);
-                if (s < NV / 2)
-                {
-                    #pragma unroll
-                    for (int e = 0; e < 8; ++e) vt[(s * 32 + g * 8 + e) * LM_VS + u * 16 + c] = kf[u][s].e[e];
-                }
+                #pragma unroll
+                for (int e = 0; e < 8; ++e) vt[(col_of[i] + e) * LM_VS + u * 16 + c] = kf[u][i].e[e];
             }
         }
         __syncthreads();
+        f32x4 sc[2];
+        #pragma unroll
+        for (int u = 0; u < 2; ++u)
+            sc[u] = (*(const f32x4*) sp[0][u][lane] + *(const f32x4*) sp[1][u][lane]) + (*(const f32x4*) sp[2][u][lane] + *(const f32x4*) sp[3][u][lane]);
         float mx = -INFINITY;
         #pragma unroll
         for (int u = 0; u < 2; ++u)
@@ -265,22 +280,23 @@ __global__ __launch_bounds__(64) void latent_decode_mfma_kernel(float* __restric
         #pragma unroll
         for (int i = 0; i < 4; ++i) { pb[i] = (__bf16) sc[0][i]; pb[4 + i] = (__bf16) sc[1][i]; }
         #pragma unroll
-        for (int t = 0; t < NV; ++t)
+        for (int t = 0; t < NVW; ++t)
         {
             acc[t] *= corr;
+            const uint16_t* vr = vt + ((w * NVW + t) * 16 + c) * LM_VS;
             union { bf16x8 v; bf16x4 h[2]; } va;
-            va.h[0] = *(const bf16x4*) (vt + (t * 16 + c) * LM_VS + g * 4);
-            va.h[1] = *(const bf16x4*) (vt + (t * 16 + c) * LM_VS + 16 + g * 4);
+            va.h[0] = *(const bf16x4*) (vr + g * 4);
+            va.h[1] = *(const bf16x4*) (vr + 16 + g * 4);
             acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va.v, pb, acc[t], 0, 0, 0);
         }
     }
     l += __shfl_xor(l, 16, 64);
     l += __shfl_xor(l, 32, 64);
     if (!head_ok) return;
-    if (g == 0) { part_ml[pidx * 2] = m; part_ml[pidx * 2 + 1] = l; }
-    float* po = part_o + pidx * (NV * 16);
+    if (w == 0 && g == 0) { part_ml[pidx * 2] = m; part_ml[pidx * 2 + 1] = l; }
+    float* po = part_o + pidx * (NV * 16) + w * NVW * 16;
     #pragma unroll
-    for (int t = 0; t < NV; ++t) *(f32x4*) (po + t * 16 + g * 4) = acc[t];          // acc[t][i] = latent column t*16 + 4g + i of head c
+    for (int t = 0; t < NVW; ++t) *(f32x4*) (po + t * 16 + g * 4) = acc[t];          // acc[t][i] = latent column (w NVW + t) * 16 + 4g + i of head c
 }
 
 // o_lat[n][h] = sum_s e^(m_s - M) O_s / (sum_s e^(m_s - M) l_s + e^(sink - M)), M = max(m_s, sink); splits without keys weigh nothing (their sums are
@@ -341,7 +357,7 @@ extern "C" int exl3_mix_latent_decode_mfma(void* o_lat, int64_t o_row, int64_t o
     MIX_CHECK(n >= 0 && n <= 65535 && heads > 0 && dim >= 0 && window > 0 && splits > 0 && splits <= 65535, "mix_latent_decode_mfma: bad sizes");
     MIX_CHECK(rank > 0 && rank <= 512 && rank % 8 == 0 && rot_dim >= 0 && rot_dim % 8 == 0, "mix_latent_decode_mfma: rank %d and rot_dim %d must be multiples of 8, rank <= 512", rank, rot_dim);
     const int nv = rank <= 128 ? 8 : (rank <= 256 ? 16 : 32);
-    MIX_CHECK(rank + rot_dim <= (nv / 2 + 2) * 32, "mix_latent_decode_mfma: rot_dim %d too large beside rank %d", rot_dim, rank);
+    MIX_CHECK(rank + rot_dim <= (nv / 2 + LM_WAVES) * 32, "mix_latent_decode_mfma: rot_dim %d too large beside rank %d", rot_dim, rank);
     MIX_CHECK((uintptr_t) ring % 16 == 0 && q_ld >= (int64_t) heads * (dim + rot_dim), "mix_latent_decode_mfma: the ring must be 16-byte aligned");
     if (n == 0) return EXL3_MIX_OK;
     const int keys_per_split = (((window + splits - 1) / splits) + LM_KEYS - 1) / LM_KEYS * LM_KEYS;
@@ -350,7 +366,7 @@ extern "C" int exl3_mix_latent_decode_mfma(void* o_lat, int64_t o_row, int64_t o
     float* part_o = scratch;
     float* part_ml = scratch + (int64_t) n * splits * heads * rp;
     const dim3 grid(splits, (heads + 15) / 16, n);
-    #define LM_LAUNCH(NVV) hipLaunchKernelGGL((latent_decode_mfma_kernel<NVV, NVV / 2 + 2>), grid, dim3(64), 0, (hipStream_t) stream, part_o, part_ml, (const bf16_t*) q_lat, ql_row, \
+    #define LM_LAUNCH(NVV) hipLaunchKernelGGL((latent_decode_mfma_kernel<NVV>), grid, dim3(64 * LM_WAVES), 0, (hipStream_t) stream, part_o, part_ml, (const bf16_t*) q_lat, ql_row, \
                                               ql_head, (const bf16_t*) q, q_ld, (const bf16_t*) ring, slots, len_after, heads, dim, rot_dim, rank, scale, window, keys_per_split, q_vec)
     if (nv == 8) LM_LAUNCH(8); else if (nv == 16) LM_LAUNCH(16); else LM_LAUNCH(32);
     #undef LM_LAUNCH

@@ -358,30 +358,31 @@ def latent_fill_k(k: torch.Tensor, ckr: torch.Tensor, heads: int, dim: int, rot_
     _check(_lib.mixlib().exl3_mix_latent_fill_k(_p(k), _view(k, heads * (dim + rot_dim), "k"), _p(ckr), n, heads, dim, rot_dim, rank, code(k.dtype), _stream(k)))
 
 
-# decode steps on the matrix cores: the cached rows of a sequence are split so that about this many one-wave workgroups are in flight (four fit a CU)
-LATENT_MFMA_TARGET_WAVES = 1024
+# decode steps on the matrix cores: the cached rows of a sequence are split so that about this many workgroups are in flight (three fit a CU), and no
+# split is shorter than two 32-key tiles (every split costs a partial sum as large as 58 cached rows, and a term in the merge)
+LATENT_MFMA_TARGET_WAVES = 512
 
 
 def latent_mfma_ok(dtype, rank: int, rot_dim: int) -> bool:
-    return dtype == torch.bfloat16 and rank % 8 == 0 and rot_dim % 8 == 0 and rank <= 512 and rot_dim <= 64
+    return dtype == torch.bfloat16 and rank % 8 == 0 and rot_dim % 8 == 0 and rank <= 512 and rot_dim <= 128
 
 
 def latent_decode(o_lat: torch.Tensor, q_lat: torch.Tensor, q_view: torch.Tensor, ring: torch.Tensor, sink, slots, len_after, dim: int, rot_dim: int, scale: float,
                   mfma: bool | None = None):
     """o_lat, q_lat: [heads, n, rank] (any strides with a unit last one); q_view [n, heads * (dim + rot_dim)] holds the rotated parts.
-    mfma None: the matrix-core kernel where it applies (bfloat16, rank and rot_dim multiples of 8, rank <= 512, rot_dim <= 64)."""
+    mfma None: the matrix-core kernel where it applies (bfloat16, rank and rot_dim multiples of 8, rank <= 512, rot_dim <= 128)."""
     heads, n, rank = q_lat.shape
     n_slots, window, row = ring.shape
     if mfma is None:
         mfma = latent_mfma_ok(o_lat.dtype, rank, rot_dim)
     if mfma:
-        _req(latent_mfma_ok(o_lat.dtype, rank, rot_dim), "latent_decode: the matrix-core kernel takes bfloat16, rank and rot_dim multiples of 8, rank <= 512, rot_dim <= 64")
+        _req(latent_mfma_ok(o_lat.dtype, rank, rot_dim), "latent_decode: the matrix-core kernel takes bfloat16, rank and rot_dim multiples of 8, rank <= 512, rot_dim <= 128")
         _req(o_lat.shape == q_lat.shape and o_lat.stride(2) == 1 and q_lat.stride(2) == 1 and row == rank + rot_dim and ring.is_contiguous(), "latent_decode: shapes")
         _req(o_lat.dtype == q_lat.dtype == q_view.dtype == ring.dtype and slots.numel() == n and len_after.numel() == n and q_view.shape[0] == n, "latent_decode: types / rows")
         if sink is not None:
             _f32c(sink, "sink"); _req(sink.numel() == heads, "latent_decode: sink")
         groups = (heads + 15) // 16
-        splits = max(1, min(LATENT_MFMA_TARGET_WAVES // max(1, n * groups), (window + 31) // 32))
+        splits = max(1, min(LATENT_MFMA_TARGET_WAVES // max(1, n * groups), (window + 63) // 64))
         rp = 128 if rank <= 128 else (256 if rank <= 256 else 512)
         scratch = torch.empty(n * splits * heads * (rp + 2), dtype=torch.float32, device=o_lat.device)
         _check(_lib.mixlib().exl3_mix_latent_decode_mfma(_p(o_lat), o_lat.stride(1), o_lat.stride(0), _p(q_lat), q_lat.stride(1), q_lat.stride(0), _p(q_view),

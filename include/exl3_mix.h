@@ -190,7 +190,7 @@ int exl3_mix_latent_decode(void* o_lat, int64_t o_row, int64_t o_head, const voi
                            int n, int heads, int dim, int rot_dim, int rank, float scale, int window, int dtype, void* stream);
 
 /* The same on the matrix cores, bfloat16 only: sixteen heads share every read of a cached row; the cached rows of a sequence are split over `splits`
- * workgroups whose partial sums a second kernel merges (the sink enters there).  rank and rot_dim multiples of 8, rank <= 512, rot_dim <= 64.  `scratch`
+ * workgroups whose partial sums a second kernel merges (the sink enters there).  rank and rot_dim multiples of 8, rank <= 512, rot_dim <= 128.  `scratch`
  * holds exl3_mix_latent_decode_mfma_scratch(...) floats. */
 int exl3_mix_latent_decode_mfma_scratch(int n, int heads, int rank, int splits, int64_t* floats);
 int exl3_mix_latent_decode_mfma(void* o_lat, int64_t o_row, int64_t o_head, const void* q_lat, int64_t ql_row, int64_t ql_head, const void* q, int64_t q_ld,
