@@ -261,15 +261,19 @@ class LatentAttention:
         q = p["q"]
         ckr = torch.empty((sb.n, rank + r), dtype=self.dtype, device=h.device)
         mix_ops.latent_prep(ckr, state["ring"], p["dkv"], self.c_norm, q, sb.tok_seq, sb.tok_pos, sb.slots, sb.len_after, self.freq, self.rot_mag, self.eps, H, d, r, rank)
-        out = torch.empty((sb.n, H * dv), dtype=self.dtype, device=h.device)
         if sb.decode:
             q_heads = q.as_strided((H, sb.n, d), (self.qk, q.stride(0), 1), q.storage_offset())
             q_lat = torch.bmm(q_heads, self.w_uk_heads)                          # [H, n, rank]
             o_lat = torch.empty_like(q_lat)
             mix_ops.latent_decode(o_lat, q_lat, q, state["ring"], self.sink, sb.slots, sb.len_after, d, r, self.scale)
             o = torch.bmm(o_lat, self.w_uv_heads_t)                              # [H, n, vdim]
-            mix_ops.heads_gate(out, o, dv, sb.n * dv, p.get("g"), H, dv)
+            if sb.n == 1 and not self.has_gate:
+                out = o.view(1, H * dv)                                          # one row: head-major is token-major
+            else:
+                out = torch.empty((sb.n, H * dv), dtype=self.dtype, device=h.device)
+                mix_ops.heads_gate(out, o, dv, sb.n * dv, p.get("g"), H, dv)
         else:
+            out = torch.empty((sb.n, H * dv), dtype=self.dtype, device=h.device)
             c = ckr[:, :rank]
             k = F.linear(c, self.w_uk_padded)                                    # [n, H * (d + r)], the rotated slots still zero
             v = F.linear(c, self.w_uv).view(sb.n, H, dv)
