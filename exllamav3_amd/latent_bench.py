@@ -3,7 +3,7 @@
 Dynamic Tanh, token side input; random weights) at sizes that resemble real models' layers, beside the closest existing model -- Vofanex layers
 (sliding-window sink attention with PolyNorm feed-forward or softmax-routed experts) of the same width / ff / expert shape, timed in the same process --
 and each kernel of the design alone against its roofline, next to the like kernel of the closest model.  Prints one JSON line; the default workload of
-bench.py and its contract are untouched.
+bench.py and the JSON line it prints are untouched.
 """
 from __future__ import annotations
 import json
