@@ -395,6 +395,35 @@ def test_sigmoid_routed_clamped_experts(gpu, dtype, n):
     assert rel(y, want) < TOL[dtype]
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_token_side_input(gpu, dtype):
+    """The per-layer token input alone: gate on the stream, the layer's slice of the token's second embedding row, projection; and its RMS-normed update."""
+    from exllamav3_amd import mix_ops
+    from exllamav3_amd.modules import TokenSide, update_residual
+    from exllamav3_amd.state_cache import StepBatch
+    g = torch.Generator().manual_seed(11)
+    width, dim, layers, layer, vocab, n = 72, 12, 3, 1, 30, 13
+    lin = lambda o, i: (torch.randn(o, i, generator=g) / math.sqrt(i)).to(torch.bfloat16)
+    Wt = {"l1.side.gate": lin(dim, width), "l1.side.proj": lin(width, dim), "l1.side.norm": (0.5 + 0.1 * torch.randn(width, generator=g)).to(torch.bfloat16),
+          "side.embed": torch.randn(vocab, dim * layers, generator=g).to(torch.bfloat16)}
+
+    class Stc:
+        def get_tensor(self, key, device="cpu"):
+            return Wt[key]
+    side = TokenSide(width, dim, layer, 1e-5)
+    side.load(Stc(), "l1.side.", Wt["side.embed"].to(dtype).to(gpu), dtype, gpu)
+    toks = torch.randint(0, vocab, (n,), generator=g)
+    x0 = torch.randn(n, width, generator=g)
+    xc = x0.to(dtype)                                          # what the gate reads: the stream in the activation type
+    sb = StepBatch(n=n, batch=1, decode=False, max_rows=n, tokens=toks.int().to(gpu), cu=None, tok_seq=None, tok_pos=None, slots=None, pos0=None, len_after=None)
+    y = side.forward(xc.to(gpu), sb)
+    x = x0.to(gpu).clone()
+    update_residual(x, y, None, rms_w=side.norm_w, eps=1e-5)
+    W64 = {k: v.to(F64) for k, v in Wt.items()}
+    want = x0.to(F64) + zo.token_side(xc.to(F64), toks, W64, "l1.", layer, dim, 1e-5)
+    assert rel(x - x0.to(gpu), want - x0.to(F64)) < TOL[dtype]
+
+
 # ---- whole models ---------------------------------------------------------------------------------------------------------------------------------
 
 @pytest.mark.parametrize("name", list(MODELS))
@@ -513,6 +542,15 @@ def test_matrix_core_prefill_long_prompt_bfloat16(gpu, zoo):
             assert float(e.max()) < TOL[dt] if dt == torch.float32 else float(e.median()) < 6e-2
 
 
+def test_a_step_that_continues_by_several_tokens_is_refused(gpu, zoo):
+    cfg, W, models = zoo["one_pass"]
+    m = models[torch.float32]
+    cache = m.new_cache(); s = cache.alloc()
+    m.step(cache.begin_step([(s, [1, 2, 3])]), cache)
+    with pytest.raises(RuntimeError):
+        cache.begin_step([(s, [4, 5])])
+
+
 def test_window_edge_shows_in_the_logits(gpu, zoo):
     """Changing the token that lies exactly `window` back from the last one (outside every layer's reach through ONE layer run) must leave a one-layer
     model's last logits unchanged, and changing the one at window - 1 must change them: in a prompt and in decoding."""
@@ -592,7 +630,7 @@ def test_matrix_core_latent_decode_batches_and_splits(gpu, H, r, rank, W, lens):
     q_lat = (torch.randn(H, B, rank, generator=g) * 0.3).to(torch.bfloat16)
     q = torch.randn(B, H * (d + r), generator=g).to(torch.bfloat16)
     sink = torch.randn(H, generator=g)
-    for sk in (None, sink):
+    for sk in (None, sink, sink + 9.0):                       # no sink, one among the scores, one that takes most of the weight
         want = torch.stack([torch.stack([absorbed_reference(q_lat[h, b].to(F64), q[b].view(H, d + r)[h, d:].to(F64), rows[b], 0.2, None if sk is None else sk[h].to(F64))
                                          for b in range(B)]) for h in range(H)])
         for target in (1, 7, 64, 4096):
